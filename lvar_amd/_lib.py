@@ -1,0 +1,62 @@
+"""ctypes binding of the C ABI declared in ``include/lvar_sparse_attn.h``.
+
+The library is loaded from the source tree; there is no fallback path: if it is missing
+the import of the operator module fails with instructions to build it.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+from .build import LIB_PATH
+
+EXPORTED_SYMBOLS = (
+    "lvar_version", "lvar_target_arch", "lvar_status_string",
+    "lvar_dense_attn_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_block_sparse_attn_fwd",
+)
+
+
+class LvarTensor(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("stride_b", C.c_int64), ("stride_h", C.c_int64), ("stride_row", C.c_int64)]
+
+
+class LvarError(RuntimeError):
+    def __init__(self, status: int, where: str, text: str):
+        super().__init__(f"{where} failed with status {status}: {text}")
+        self.status = status
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m lvar_amd.build` (needs hipcc). "
+            "lvar_amd has no CPU or PyTorch fallback.")
+    lib = C.CDLL(LIB_PATH)
+    T, P, I, I64, F = LvarTensor, C.c_void_p, C.c_int, C.c_int64, C.c_float
+    lib.lvar_version.restype = I
+    lib.lvar_version.argtypes = []
+    lib.lvar_target_arch.restype = C.c_char_p
+    lib.lvar_target_arch.argtypes = []
+    lib.lvar_status_string.restype = C.c_char_p
+    lib.lvar_status_string.argtypes = [I]
+    lib.lvar_dense_attn_fwd.restype = I
+    lib.lvar_dense_attn_fwd.argtypes = [T, T, T, T, P, P, I, I, I, I, I, F, P]
+    lib.lvar_colsum_fwd.restype = I
+    lib.lvar_colsum_fwd.argtypes = [T, T, P, P, P, I, I, I, I, I, I, F, P]
+    lib.lvar_csp_attn_fwd.restype = I
+    lib.lvar_csp_attn_fwd.argtypes = [T, T, T, T, T, P, P, P, P, I, I64, I, I, I, I, I, I, F, F, P]
+    lib.lvar_block_sparse_attn_fwd.restype = I
+    lib.lvar_block_sparse_attn_fwd.argtypes = [T, T, T, T, P, P, P, I64, I64, P, I64, I64, I64, I, I, I, I, I, I, I, I, F, P]
+    _lib = lib
+    return lib
+
+
+def check(status: int, where: str) -> None:
+    if status != 0:
+        raise LvarError(status, where, load().lvar_status_string(status).decode())

@@ -1,0 +1,138 @@
+// extern "C" entry points declared in include/lvar_sparse_attn.h: argument validation and
+// parameter packing; all device work is in attn_fwd.hip / colsum.hip.
+#include <cmath>
+#include <cstdlib>
+#include "../../include/lvar_sparse_attn.h"
+#include "launch.h"
+
+using namespace lvar;
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// rows are read/written with 16-byte vector accesses: base and every stride must keep them aligned
+bool view_ok(const lvar_tensor_t& t) {
+  return t.ptr && aligned16(t.ptr) && t.stride_b % 8 == 0 && t.stride_h % 8 == 0 && t.stride_row % 8 == 0;
+}
+
+bool shape_ok(int B, int H, int Lq, int Lk, float scale) {
+  return B > 0 && H > 0 && Lq > 0 && Lk > 0 && std::isfinite(scale) && scale > 0.f;
+}
+
+int gather_waves() {
+  static int v = [] {
+    const char* e = std::getenv("LVAR_CSP_WAVES");
+    int n = e ? std::atoi(e) : 6;
+    return (n == 2 || n == 3 || n == 6) ? n : 6;
+  }();
+  return v;
+}
+
+void fill_qkv(AttnParams& p, const lvar_tensor_t& q, const lvar_tensor_t& k, const lvar_tensor_t& v) {
+  p.q = (const bf16_t*)q.ptr; p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sr = q.stride_row;
+  p.k = (const bf16_t*)k.ptr; p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sr = k.stride_row;
+  p.v = (const bf16_t*)v.ptr; p.v_sb = v.stride_b; p.v_sh = v.stride_h; p.v_sr = v.stride_row;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lvar_version(void) { return 100; }
+const char* lvar_target_arch(void) { return "gfx950"; }
+
+const char* lvar_status_string(int status) {
+  switch (status) {
+    case LVAR_OK: return "ok";
+    case LVAR_EINVAL: return "invalid argument (size, null/misaligned pointer, stride or scale)";
+    case LVAR_EUNSUPPORTED: return "unsupported head_dim or block shape";
+    case LVAR_ELAUNCH: return "HIP launch failed";
+    default: return "unknown status";
+  }
+}
+
+int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+                        int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
+  if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k)) return LVAR_EINVAL;
+  const bool lse_only = (o.ptr == nullptr);
+  if (!lse_only && (!view_ok(v) || !view_ok(o))) return LVAR_EINVAL;
+  if (lse_only && !(M && L)) return LVAR_EINVAL;
+  AttnParams p{};
+  fill_qkv(p, q, k, lse_only ? k : v);
+  p.o = (bf16_t*)o.ptr; p.o_sb = o.stride_b; p.o_sh = o.stride_h; p.o_sr = o.stride_row;
+  p.M = M; p.L = L;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
+  p.c = scale * kLog2e; p.o_scale = 1.f;
+  return launch_attn(p, head_dim, MODE_DENSE, false, lse_only, 4, (hipStream_t)stream);
+}
+
+int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* M, const float* L, float* cs,
+                    int B, int H, int Lq, int Lk, int head_dim, int q_group_size, float scale, void* stream) {
+  if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !M || !L || !cs) return LVAR_EINVAL;
+  if (q_group_size <= 0 || q_group_size % 32 != 0) return LVAR_EINVAL;
+  ColsumParams p{};
+  p.q = (const bf16_t*)q.ptr; p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sr = q.stride_row;
+  p.k = (const bf16_t*)k.ptr; p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sr = k.stride_row;
+  p.M = M; p.L = L; p.cs = cs;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
+  p.group_rows = q_group_size;
+  p.G = (Lq + q_group_size - 1) / q_group_size;
+  p.c = scale * kLog2e;
+  return launch_colsum(p, head_dim, (hipStream_t)stream);
+}
+
+int lvar_csp_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o_accum, lvar_tensor_t o,
+                      float* M, float* L, const int32_t* indices, const int32_t* counts, int G,
+                      int64_t idx_row_stride, int group_rows, int B, int H, int Lq, int Lk, int head_dim,
+                      float o_scale, float scale, void* stream) {
+  if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
+  if (o_accum.ptr && !view_ok(o_accum)) return LVAR_EINVAL;
+  if (!indices || !counts || G <= 0 || idx_row_stride <= 0) return LVAR_EINVAL;
+  if (group_rows <= 0 || group_rows % 32 != 0 || (int64_t)G * group_rows < Lq) return LVAR_EINVAL;
+  AttnParams p{};
+  fill_qkv(p, q, k, v);
+  p.o = (bf16_t*)o.ptr; p.o_sb = o.stride_b; p.o_sh = o.stride_h; p.o_sr = o.stride_row;
+  p.o_accum = (const bf16_t*)o_accum.ptr; p.oa_sb = o_accum.stride_b; p.oa_sh = o_accum.stride_h; p.oa_sr = o_accum.stride_row;
+  p.M = M; p.L = L;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
+  p.c = scale * kLog2e; p.o_scale = o_scale;
+  p.list = indices; p.cnt = counts;
+  p.list_sg = idx_row_stride; p.list_sh = (int64_t)G * idx_row_stride; p.list_sb = (int64_t)H * p.list_sh;
+  p.cnt_sh = G; p.cnt_sb = (int64_t)H * G;
+  p.list_len = (int)(idx_row_stride > 0x7fffffff ? 0x7fffffff : idx_row_stride);
+  p.group_rows = group_rows;
+  int nw = gather_waves();
+  while (group_rows % (nw * 32) != 0) nw = (nw == 6) ? 3 : (nw == 3 ? 2 : 1);
+  if (nw == 1) {
+    if (group_rows % 64 == 0) nw = 2; else return LVAR_EUNSUPPORTED;
+  }
+  return launch_attn(p, head_dim, MODE_GATHER, true, false, nw, (hipStream_t)stream);
+}
+
+int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+                               const int32_t* kv_num_blocks, int64_t stride_nb_b, int64_t stride_nb_h,
+                               const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
+                               int64_t stride_ki_q, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
+                               int head_dim, float scale, void* stream) {
+  if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
+  if (!kv_num_blocks || !kv_indices || nk_max <= 0) return LVAR_EINVAL;
+  if (block_q != 128 || (block_k != 64 && block_k != 128)) return LVAR_EUNSUPPORTED;
+  AttnParams p{};
+  fill_qkv(p, q, k, v);
+  p.o = (bf16_t*)o.ptr; p.o_sb = o.stride_b; p.o_sh = o.stride_h; p.o_sr = o.stride_row;
+  p.M = M; p.L = L;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
+  p.c = scale * kLog2e; p.o_scale = 1.f;
+  p.list = kv_indices; p.cnt = kv_num_blocks;
+  p.list_sb = stride_ki_b; p.list_sh = stride_ki_h; p.list_sg = stride_ki_q;
+  p.cnt_sb = stride_nb_b; p.cnt_sh = stride_nb_h;
+  p.list_len = nk_max;
+  p.group_rows = block_q;
+  p.sub_shift = (block_k == 128) ? 1 : 0;
+  return launch_attn(p, head_dim, MODE_BLOCK, false, false, 4, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,51 @@
+// Host-side launch interface shared by the kernel translation units and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "common.h"
+#include "../../include/lvar_sparse_attn.h"
+
+namespace lvar {
+
+enum { MODE_DENSE = 0, MODE_BLOCK = 1, MODE_GATHER = 2 };
+
+struct AttnParams {
+  const bf16_t *q, *k, *v;
+  bf16_t* o;
+  const bf16_t* o_accum;
+  float *M, *L;
+  int64_t q_sb, q_sh, q_sr;
+  int64_t k_sb, k_sh, k_sr;
+  int64_t v_sb, v_sh, v_sr;
+  int64_t o_sb, o_sh, o_sr;
+  int64_t oa_sb, oa_sh, oa_sr;
+  int B, H, Lq, Lk;
+  float c;        // softmax scale * log2(e)
+  float o_scale;  // epilogue factor of the token-list variant
+  // key-tile list: kv_indices / kv_num_blocks (block list) or indices / counts (token list)
+  const int32_t* list;
+  const int32_t* cnt;
+  int64_t list_sb, list_sh, list_sg;
+  int64_t cnt_sb, cnt_sh;
+  int list_len;    // entries available per list row; counts are clamped to it
+  int group_rows;  // query rows sharing one list
+  int sub_shift;   // log2(64-key tiles per key block)
+  int nqt, total_wg;
+};
+
+struct ColsumParams {
+  const bf16_t *q, *k;
+  const float *M, *L;
+  float* cs;
+  int64_t q_sb, q_sh, q_sr;
+  int64_t k_sb, k_sh, k_sr;
+  int B, H, Lq, Lk, G;
+  int group_rows;
+  float c;
+  int nkt, total_wg;
+};
+
+int launch_attn(const AttnParams& p, int head_dim, int mode, bool accum, bool lse_only, int nwaves, hipStream_t s);
+int launch_colsum(const ColsumParams& p, int head_dim, hipStream_t s);
+
+}  // namespace lvar

@@ -1,0 +1,245 @@
+"""Operator API of the sparse-attention path, signature-compatible with the reference's
+``kernels/sparse_attn/sparse_attn_ops.py`` (``dense_attn`` :21-59, ``dense_colsum_attn_s`` :65-113,
+``dense_colsum_attn_q`` :119-149, ``csp_attn`` :273-292) and with the kernel-level functions of
+``kernels/sparse_attn/triton/__init__.py`` (``dense_colsum_attn``, ``csp_attn_delta``).
+
+Tensor contract: q ``[B,H,Lq,d]``, k/v ``[B,H,Lk,d]`` bf16 on a HIP device, unit stride on d;
+``cs`` fp32 ``[B,H,ceil(Lq/bm),Lk]``; ``indices`` int32 ``[B,H,G,Lk]`` (valid prefix ``counts``),
+``counts`` int32 ``[B,H,G]``; ``(M, L)`` fp32 ``[B,H,Lq,1]`` in the base-2 convention
+``M = max(qk*scale*log2e)``, ``L = sum exp2(qk*scale*log2e - M)``.  Outputs are freshly allocated;
+inputs are never written.  Work is enqueued on the current torch stream of the tensors' device.
+
+All compute runs in the HIP library; there is no PyTorch or CPU fallback.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from .sparse_attn_config import get_kernel_config_attn
+
+__all__ = [
+    "dense_attn", "dense_colsum_attn", "dense_colsum_attn_s", "dense_colsum_attn_q", "colsum",
+    "csp_attn", "csp_attn_delta", "block_sparse_attn", "ShapeError",
+]
+
+
+class ShapeError(AssertionError, ValueError):
+    """Shape / dtype contract violation (the reference raises AssertionError at the same places)."""
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ShapeError(msg)
+
+
+def _scale(q: torch.Tensor, scale) -> float:
+    return 1.0 / math.sqrt(q.shape[-1]) if scale is None else float(scale)
+
+
+def _prep(t: torch.Tensor, name: str) -> torch.Tensor:
+    _require(t.dim() == 4, f"{name} must be [B,H,L,d], got {tuple(t.shape)}")
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on a HIP device; lvar_amd has no CPU path")
+    if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]) or t.data_ptr() % 16:
+        t = t.contiguous()
+    return t
+
+
+def _view(t: Optional[torch.Tensor]) -> _lib.LvarTensor:
+    if t is None:
+        return _lib.LvarTensor(None, 0, 0, 0)
+    return _lib.LvarTensor(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def _check_qkv(q, k, v):
+    _require(k.shape == v.shape, f"k/v shape mismatch: {tuple(k.shape)} vs {tuple(v.shape)}")
+    _require(q.shape[0] == k.shape[0] and q.shape[1] == k.shape[1] and q.shape[3] == k.shape[3],
+             f"q/k batch, head or head_dim mismatch: {tuple(q.shape)} vs {tuple(k.shape)}")
+    _require(q.shape[-1] in (64, 128), f"head_dim must be 64 or 128, got {q.shape[-1]}")
+    _require(q.device == k.device == v.device, "q, k, v must be on the same device")
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def dense_attn(q, k, v, scale=None):
+    """Dense flash attention, ``(o, (M, L))`` (reference ``dense_attn``, sparse_attn_ops.py:21-59,
+    Triton-provider return convention: ``lse`` is the tuple ``(M, L)``, each ``[B,H,Lq,1]``)."""
+    q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
+    _check_qkv(q, k, v)
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device)
+    M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
+    L = torch.empty_like(M)
+    with torch.cuda.device(q.device):
+        st = _lib.load().lvar_dense_attn_fwd(_view(q), _view(k), _view(v), _view(o), M.data_ptr(), L.data_ptr(),
+                                            B, H, Lq, Lk, d, _scale(q, scale), _stream(q))
+    _lib.check(st, "lvar_dense_attn_fwd")
+    return o, (M, L)
+
+
+def _lse_only(q, k, scale):
+    B, H, Lq, d = q.shape
+    M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
+    L = torch.empty_like(M)
+    with torch.cuda.device(q.device):
+        st = _lib.load().lvar_dense_attn_fwd(_view(q), _view(k), _view(None), _view(None), M.data_ptr(), L.data_ptr(),
+                                            B, H, Lq, k.shape[2], d, _scale(q, scale), _stream(q))
+    _lib.check(st, "lvar_dense_attn_fwd")
+    return M, L
+
+
+def _colsum_given_lse(q, k, M, L, scale, q_group_size):
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    G = (Lq + q_group_size - 1) // q_group_size
+    cs = torch.empty((B, H, G, Lk), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        st = _lib.load().lvar_colsum_fwd(_view(q), _view(k), M.data_ptr(), L.data_ptr(), cs.data_ptr(),
+                                        B, H, Lq, Lk, d, q_group_size, _scale(q, scale), _stream(q))
+    _lib.check(st, "lvar_colsum_fwd")
+    return cs
+
+
+def colsum(q, k, scale=None, q_group_size: Optional[int] = None, lse: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
+    """Column sums of the softmax probabilities per group of ``q_group_size`` query rows
+    (default: the kernel config's ``bm`` = 192), fp32 ``[B,H,G,Lk]``.  Self-contained two-pass form
+    (statistics sweep, then column sweep) unless ``lse=(M, L)`` from a previous dense pass is given."""
+    q, k = _prep(q, "q"), _prep(k, "k")
+    _check_qkv(q, k, k)
+    if q_group_size is None:
+        q_group_size = get_kernel_config_attn()["bm"]
+    _require(q_group_size > 0 and q_group_size % 32 == 0, "q_group_size must be a positive multiple of 32")
+    if lse is None:
+        M, L = _lse_only(q, k, scale)
+    else:
+        M, L = (t.to(torch.float32).contiguous() for t in lse)
+        _require(M.numel() == q.shape[0] * q.shape[1] * q.shape[2] == L.numel(), "lse must be ([B,H,Lq,1], [B,H,Lq,1])")
+    return _colsum_given_lse(q, k, M, L, scale, q_group_size)
+
+
+def dense_colsum_attn(q, k, v, scale=None):
+    """Kernel-level op ``(o, blocksums, (M, L))`` (reference Triton ``dense_colsum_attn``,
+    kernels/sparse_attn/triton/attn_dense_colsum.py:237-296): dense attention, then the column
+    sweep that reuses its (M, L)."""
+    q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
+    o, (M, L) = dense_attn(q, k, v, scale)
+    cs = _colsum_given_lse(q, k, M, L, scale, get_kernel_config_attn()["bm"])
+    return o, cs, (M, L)
+
+
+def dense_colsum_attn_s(q, k, v, scale=None):
+    """``(o, cs)`` (reference ``dense_colsum_attn_s``, sparse_attn_ops.py:65-113)."""
+    o, cs, (M, L) = dense_colsum_attn(q, k, v, scale)
+    pad_to = get_kernel_config_attn()["bm"]
+    assert M.shape == (q.shape[0], q.shape[1], q.shape[2], 1), "L shape mismatch"
+    assert o.shape == q.shape, "Output shape mismatch"
+    assert cs.shape == (q.shape[0], q.shape[1], (q.shape[-2] + pad_to - 1) // pad_to, k.shape[2]), "CS shape mismatch"
+    return o, cs
+
+
+def dense_colsum_attn_q(q, k, v, scale=None):
+    """``(o, cs)`` (reference ``dense_colsum_attn_q``, sparse_attn_ops.py:119-149).  The reference
+    keeps a separate "quality" variant because its CUDA colsum is bf16 and ignores ``scale``; here
+    both variants are the same fp32, scale-honouring kernels."""
+    return dense_colsum_attn_s(q, k, v, scale)
+
+
+def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats):
+    q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
+    _check_qkv(q, k, v)
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    bm = get_kernel_config_attn()["bm"]
+    _require(indices.dim() == 4 and indices.shape[0] == B and indices.shape[1] == H,
+             f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}")
+    G = indices.shape[2]
+    _require(G * bm >= Lq, f"indices has {G} query groups of {bm} rows, fewer than Lq={Lq}")
+    _require(tuple(counts.shape) == tuple(indices.shape[:-1]),
+             f"Indices counts shape mismatch - indices_counts: {tuple(counts.shape)}, indices: {tuple(indices.shape)}")
+    if indices.dtype != torch.int32 or counts.dtype != torch.int32:
+        raise TypeError("indices and indices_counts must be int32")
+    _require(indices.device == q.device and counts.device == q.device, "indices / counts must be on q's device")
+    if indices.stride(3) != 1 or indices.stride(1) != G * indices.stride(2) or indices.stride(0) != H * indices.stride(1):
+        indices = indices.contiguous()
+    counts = counts.contiguous()
+    if o_accum is not None:
+        o_accum = _prep(o_accum, "o")
+        _require(o_accum.shape == q.shape, f"Output shape mismatch - o: {tuple(o_accum.shape)}, q: {tuple(q.shape)}")
+    o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device)
+    M = L = None
+    if want_stats:
+        M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
+        L = torch.empty_like(M)
+    with torch.cuda.device(q.device):
+        st = _lib.load().lvar_csp_attn_fwd(_view(q), _view(k), _view(v), _view(o_accum), _view(o), _ptr(M), _ptr(L),
+                                          indices.data_ptr(), counts.data_ptr(), G, indices.stride(2), bm,
+                                          B, H, Lq, Lk, d, float(o_scale), _scale(q, scale), _stream(q))
+    _lib.check(st, "lvar_csp_attn_fwd")
+    return o, M, L
+
+
+def csp_attn(q, k, v, scale, indices, indices_counts, o, o_scale):
+    """``o + o_scale * softmax(q k[idx]^T scale) v[idx]`` with per-192-row-group key-token lists
+    (reference ``csp_attn``, sparse_attn_ops.py:273-292).  Returns a new tensor; ``o`` is not
+    modified (the reference's Triton behaviour).  The sum is formed in fp32 and rounded once."""
+    _require(indices.dim() == 4 and indices.shape[-1] == k.shape[-2] and indices.shape[:2] == q.shape[:2],
+             f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}, k: {tuple(k.shape)}")
+    _require(tuple(o.shape) == tuple(q.shape), f"Output shape mismatch - o: {tuple(o.shape)}, q: {tuple(q.shape)}")
+    out, _, _ = _csp_launch(q, k, v, indices, indices_counts, o, o_scale, scale, False)
+    return out
+
+
+def csp_attn_delta(q, k, v, sparsity_indices, sparsity_counts, O_scale=1.0, scale=None):
+    """Kernel-level op ``(O_scale * delta, (M, L))`` (reference Triton ``csp_attn``,
+    kernels/sparse_attn/triton/attn_csp.py:215-265, which accumulates onto zeros)."""
+    out, M, L = _csp_launch(q, k, v, sparsity_indices, sparsity_counts, None, O_scale, scale, True)
+    return out, (M, L)
+
+
+def block_sparse_attn(q, k, v, kv_num_blocks, kv_indices, block_q: int = 128, block_k: int = 64, scale=None):
+    """Block-sparse attention over a compacted per-query-block list of key blocks in the flex
+    ``BlockMask`` layout consumed by ``SparseFlexAttn`` (models/sparvar/basic_sparvar.py:55-72,187-194):
+    ``kv_num_blocks`` int32 ``[B|1,H|1,nQ]``, ``kv_indices`` int32 ``[B|1,H|1,nQ,nKmax]``.
+    Returns ``(o, (M, L))``."""
+    q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
+    _check_qkv(q, k, v)
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    _require(block_q == 128 and block_k in (64, 128), "block shape must be (128,64) or (128,128)")
+    nQ = (Lq + block_q - 1) // block_q
+    _require(kv_num_blocks.dim() == 3 and kv_indices.dim() == 4, "kv_num_blocks must be [B,H,nQ], kv_indices [B,H,nQ,nKmax]")
+    _require(kv_num_blocks.shape[2] == nQ and kv_indices.shape[2] == nQ,
+             f"block list has {kv_num_blocks.shape[2]} query blocks, expected {nQ}")
+    _require(kv_num_blocks.shape[0] in (1, B) and kv_num_blocks.shape[1] in (1, H)
+             and tuple(kv_indices.shape[:2]) == tuple(kv_num_blocks.shape[:2]), "block list batch/head dims must be 1 or B/H")
+    if kv_num_blocks.dtype != torch.int32 or kv_indices.dtype != torch.int32:
+        raise TypeError("kv_num_blocks and kv_indices must be int32")
+    kv_num_blocks = kv_num_blocks.contiguous()
+    kv_indices = kv_indices.contiguous()
+    nb_sb = kv_num_blocks.stride(0) if kv_num_blocks.shape[0] == B and B > 1 else 0
+    nb_sh = kv_num_blocks.stride(1) if kv_num_blocks.shape[1] == H and H > 1 else 0
+    ki_sb = kv_indices.stride(0) if kv_indices.shape[0] == B and B > 1 else 0
+    ki_sh = kv_indices.stride(1) if kv_indices.shape[1] == H and H > 1 else 0
+    o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device)
+    M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
+    L = torch.empty_like(M)
+    with torch.cuda.device(q.device):
+        st = _lib.load().lvar_block_sparse_attn_fwd(
+            _view(q), _view(k), _view(v), _view(o), M.data_ptr(), L.data_ptr(),
+            kv_num_blocks.data_ptr(), nb_sb, nb_sh, kv_indices.data_ptr(), ki_sb, ki_sh, kv_indices.stride(2), kv_indices.shape[3],
+            block_q, block_k, B, H, Lq, Lk, d, _scale(q, scale), _stream(q))
+    _lib.check(st, "lvar_block_sparse_attn_fwd")
+    return o, (M, L)
