@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-attention hot path on one MI355X.
+
+A "step" is one block-sparse flash-attention forward over the Infinity-2B 1024x1024 last-scale
+self-attention batch (B=2 cond+uncond, H=16, d=128, Lq=4096, Lk=10521, bf16, 128x64 blocks at 25 %
+density: keys of scales <= 16 always kept, +-2 key blocks around the query position in every later
+scale, remainder chosen by colsum top-k).  Inputs are synthetic, seeded, resident in HBM before the
+timed region.  The headline value is effective TFLOP/s over ACTIVE blocks (4*d*rows*cols per active
+block, softmax flops not counted).
+
+Prints ONE JSON line.  ``--workload`` selects the other single-GPU configurations for profiling.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X published dense bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel
+# of known size; the summaries are under profiles/.  None = not measured for that workload.
+MEASURED_TRAFFIC = {}
+
+
+def make_qkv(B, H, Lq, Lk, d, seed, amp):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(B, H, Lq, d, generator=g) * amp).to(torch.bfloat16)
+    k = (torch.randn(B, H, Lk, d, generator=g) * amp).to(torch.bfloat16)
+    v = (torch.randn(B, H, Lk, d, generator=g) * amp).to(torch.bfloat16)
+    return q, k, v
+
+
+def block_flops(num, idx, Lq, Lk, d, bq, bk, B, H):
+    """4*d*sum(rows_i*cols_j) over active blocks, edge blocks clipped; lists may broadcast over B/H."""
+    nQ = num.shape[-1]
+    rows = torch.clamp(Lq - torch.arange(nQ, device=num.device) * bq, max=bq).double()
+    cols = torch.clamp(Lk - idx.long() * bk, min=0, max=bk).double()
+    valid = torch.arange(idx.shape[-1], device=num.device) < num.unsqueeze(-1)
+    per_row = (cols * valid).sum(-1) * rows
+    mult = (B // num.shape[0]) * (H // num.shape[1])
+    return 4.0 * d * float(per_row.sum().item()) * mult
+
+
+def time_launches(fn, steps, warmup):
+    """Average duration of ``steps`` back-to-back launches measured with HIP events recorded on the
+    stream the kernels are enqueued on (torch's current stream), plus host wall time."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return e0.elapsed_time(e1) / steps, wall * 1e3 / steps
+
+
+def cpu_baseline_block_sparse(q, k, v, num, idx, bq, bk, budget_s=20.0):
+    """Oracle (torch fp32 on the host cores) on a bounded sample of the same workload: whole
+    (batch, head) slices until ~budget_s of CPU time is spent.  Returns TFLOP/s and a description."""
+    import oracle
+    torch.set_num_threads(os.cpu_count() or 1)
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    done, flops, t_used = 0, 0.0, 0.0
+    for bh in range(B * H):
+        b, h = divmod(bh, H)
+        nb = num[b:b + 1, h:h + 1] if num.shape[0] > 1 else num[:, h:h + 1] if num.shape[1] > 1 else num
+        ib = idx[b:b + 1, h:h + 1] if idx.shape[0] > 1 else idx[:, h:h + 1] if idx.shape[1] > 1 else idx
+        t0 = time.perf_counter()
+        oracle.block_sparse_attn(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], nb, ib, bq, bk)
+        t_used += time.perf_counter() - t0
+        flops += block_flops(nb, ib, Lq, Lk, d, bq, bk, 1, 1)
+        done += 1
+        if t_used > budget_s:
+            break
+    return flops / t_used / 1e12, f"{done} of {B * H} (batch,head) slices of the same inputs and block lists, {t_used:.1f} s"
+
+
+def cpu_baseline_dense(q, k, v, budget_s=20.0, colsum=False):
+    import oracle
+    torch.set_num_threads(os.cpu_count() or 1)
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    done, t_used = 0, 0.0
+    for bh in range(B * H):
+        b, h = divmod(bh, H)
+        t0 = time.perf_counter()
+        if colsum:
+            oracle.dense_colsum_attn(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1])
+        else:
+            oracle.dense_attn(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1])
+        t_used += time.perf_counter() - t0
+        done += 1
+        if t_used > budget_s:
+            break
+    return done, t_used
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="block_sparse_25",
+                    help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | density_<pct> | video_10")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget-s", type=float, default=20.0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the hot path on ONE GPU; --gpus N with N > 1 is not supported "
+              "(the path shards over (batch, head) with no exchange step, see DESIGN.md).", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU fallback)", file=sys.stderr)
+        sys.exit(1)
+
+    from lvar_amd import mask_build as mb
+    from lvar_amd import sparse_attn_ops as ops
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    wl = args.workload
+    d = 128
+    aux = {}
+    cpu = None
+
+    if wl in ("block_sparse_25", "dense", "colsum", "csp") or wl.startswith("density_"):
+        B, H, Lq, Lk = (1 if wl.startswith("density_") else 2), 16, 4096, 10521
+        amp = 1.0 if (wl.startswith("density_") or wl == "colsum") else 0.5
+    elif wl == "colsum_scale48":
+        B, H, Lq, Lk, amp = 2, 16, 2304, 6425, 1.0
+    elif wl == "video_10":
+        B, H, Lq, Lk, amp = 1, 24, 32768, 32768, 0.5
+    else:
+        raise SystemExit(f"unknown workload {wl}")
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=1234, amp=amp)
+    qg, kg, vg = q.to(dev), k.to(dev), v.to(dev)
+    scale = 1.0 / math.sqrt(d)
+    dense_flops = 4.0 * B * H * Lq * Lk * d
+    config = {"workload": wl, "B": B, "H": H, "head_dim": d, "Lq": Lq, "Lk": Lk}
+
+    if wl == "block_sparse_25" or wl.startswith("density_") or wl == "video_10":
+        bq, bk = 128, (128 if wl == "video_10" else 64)
+        nQ, nK = (Lq + bq - 1) // bq, (Lk + bk - 1) // bk
+        if wl == "block_sparse_25":
+            cs = ops.colsum(qg, kg, scale, q_group_size=bq)                 # [B,H,nQ,Lk]
+            mask = mb.sink_window_topk_block_mask(mb.key_block_sums(cs, bk), bq, bk, density=0.25)
+            del cs
+            config.update({"block": [bq, bk], "mask": "sink(scales<=16)+window(+-2 blocks/scale)+colsum top-k", "density": 0.25})
+        elif wl == "video_10":
+            # 3D local window over a latent grid of 8 frames x 64 x 64 tokens (+-1 frame, +-1 spatial
+            # block) plus 2 % of blocks by colsum top-k of a strided query sample
+            blk = torch.arange(nQ, device=dev)
+            f, s = blk // 32, blk % 32                                      # 32 blocks of 128 tokens per frame
+            near = ((f[:, None] - f[None, :]).abs() <= 1) & ((s[:, None] - s[None, :]).abs() <= 1)
+            cs = ops.colsum(qg[:, :, ::8].contiguous(), kg, scale, q_group_size=32)   # 4096 sampled rows, groups of 32
+            score = mb.key_block_sums(cs, bk)[:, :, :nQ]
+            score = score.masked_fill(near[None, None], -float("inf"))
+            extra = int(round(0.02 * nK))
+            top = torch.topk(score, k=extra, dim=-1).indices
+            mask = near[None, None].expand(B, H, nQ, nK).clone()
+            mask.scatter_(-1, top, True)
+            del cs, score
+            config.update({"block": [bq, bk], "mask": "3D window (+-1 frame, +-1 spatial block) + 2% colsum top-k"})
+        else:
+            pct = float(wl.split("_")[1])
+            g = torch.Generator().manual_seed(7)
+            mask = torch.rand(B, H, nQ, nK, generator=g) < pct / 100.0
+            mask.scatter_(-1, torch.randint(0, nK, (B, H, nQ, 1), generator=g), True)
+            mask = mask.to(dev)
+            config.update({"block": [bq, bk], "mask": f"Bernoulli({pct}%) blocks, >=1 per row"})
+        num, idx = mb.block_mask_to_lists(mask)
+        flops = block_flops(num, idx, Lq, Lk, d, bq, bk, B, H)
+        config["active_block_fraction"] = round(float(mask.float().mean().item()), 4)
+        fn = lambda: ops.block_sparse_attn(qg, kg, vg, num, idx, bq, bk, scale)
+        kernel = "attn_fwd_kernel<128,4,BLOCK>"
+        if not args.no_cpu_baseline:
+            val, sample = cpu_baseline_block_sparse(q, k, v, num.cpu(), idx.cpu(), bq, bk, args.cpu_budget_s)
+            cpu = {"value": round(val, 5), "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port", "sample": sample}
+    elif wl == "dense":
+        flops = dense_flops
+        fn = lambda: ops.dense_attn(qg, kg, vg, scale)
+        kernel = "attn_fwd_kernel<128,4,DENSE>"
+        if not args.no_cpu_baseline:
+            done, t = cpu_baseline_dense(q, k, v, args.cpu_budget_s)
+            cpu = {"value": round(dense_flops / (B * H) * done / t / 1e12, 5), "unit": "TFLOP/s", "cores": os.cpu_count(),
+                   "kind": "port", "sample": f"{done} of {B * H} (batch,head) slices, {t:.1f} s"}
+    elif wl in ("colsum", "colsum_scale48"):
+        M, L = ops._lse_only(qg, kg, scale)
+        flops = 2.0 * B * H * Lq * Lk * d      # column sweep with (M, L) supplied
+        fn = lambda: ops._colsum_given_lse(qg, kg, M, L, scale, 192)
+        kernel = "colsum_kernel<128,2>"
+        config["form"] = "one-pass given (M,L): 2*B*H*Lq*Lk*d flops"
+        if not args.no_cpu_baseline:
+            done, t = cpu_baseline_dense(q, k, v, args.cpu_budget_s, colsum=True)
+            cpu = {"value": round(1.5 * dense_flops / (B * H) * done / t / 1e12, 5), "unit": "TFLOP/s", "cores": os.cpu_count(),
+                   "kind": "port", "sample": f"{done} of {B * H} (batch,head) slices of dense attention + colsum (6*Lq*Lk*d flops each), {t:.1f} s"}
+    elif wl == "csp":
+        G = (Lq + 191) // 192
+        cs = ops.colsum(qg, kg, scale)
+        inds, counts = mb.topk_index_list(cs, 0.2)
+        del cs
+        cnt = int(counts[0, 0, 0])
+        rows = torch.tensor([min(192, Lq - g * 192) for g in range(G)], dtype=torch.float64)
+        flops = 4.0 * d * B * H * float(rows.sum()) * cnt
+        o0 = torch.zeros_like(qg)
+        fn = lambda: ops.csp_attn(qg, kg, vg, scale, inds, counts, o0, 1)
+        kernel = "attn_fwd_kernel<128,6,GATHER>"
+        config.update({"top_keys": 0.2, "count": cnt})
+
+    ms, wall_ms = time_launches(fn, args.steps, args.warmup)
+    tflops = flops / (ms * 1e-3) / 1e12
+
+    if wl == "block_sparse_25":
+        # companion numbers named by the metric: colsum (+ mask build) versus the dense attention it replaces
+        dense_ms, _ = time_launches(lambda: ops.dense_attn(qg, kg, vg, scale), 10, 3)
+        M, L = ops._lse_only(qg, kg, scale)
+        cs_ms, _ = time_launches(lambda: ops._colsum_given_lse(qg, kg, M, L, scale, 128), 10, 3)
+        lse_ms, _ = time_launches(lambda: ops._lse_only(qg, kg, scale), 10, 3)
+
+        def build():
+            cs = ops._colsum_given_lse(qg, kg, M, L, scale, 128)
+            return mb.block_mask_to_lists(mb.sink_window_topk_block_mask(mb.key_block_sums(cs, 64), 128, 64, 0.25))
+        build_ms, _ = time_launches(build, 5, 2)
+        aux = {"dense_attn_ms": round(dense_ms, 4), "dense_attn_tflops": round(dense_flops / dense_ms / 1e9, 1),
+               "colsum_given_lse_us": round(cs_ms * 1e3, 1), "lse_pass_us": round(lse_ms * 1e3, 1),
+               "colsum_plus_mask_build_ms": round(build_ms, 4), "speedup_vs_dense": round(dense_ms / ms, 3)}
+
+    out = {
+        "metric": "block-sparse attn effective TFLOP/s over active blocks" if kernel.endswith("BLOCK>") else f"{wl} effective TFLOP/s",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (seeded N(0,1)*%.1f, random-init, no checkpoint)" % amp,
+        "config": config,
+        "roofline": {"bound": "mfma", "kernel": kernel, "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC.get(wl),
+                     "flops_per_launch": flops, "host_wall_ms_per_step": round(wall_ms, 5)},
+        "cpu_baseline": cpu,
+        "device": torch.cuda.get_device_name(0),
+    }
+    if aux:
+        out["aux"] = aux
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,233 @@
+"""Mask / key-list construction around the sparse-attention kernels (host-side policy code).
+
+Counterparts of the arithmetic in the reference's ``SparseDiffAttn`` and ``SparseFlexAttn``
+(models/sparvar/sparse_attn.py, models/sparvar/basic_sparvar.py); every function works on the
+device its inputs live on and is vectorised with torch, so it can run on the GPU between the
+colsum kernel and the sparse-attention kernel without a host round trip.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from .sparse_attn_config import get_kernel_config_attn
+
+INFINITY_SCALES = (1, 2, 4, 6, 8, 12, 16, 20, 24, 32, 40, 48, 64)
+
+__all__ = [
+    "INFINITY_SCALES", "scale_offsets", "indices_count", "topk_index_list", "map_inds_counts_across_scales",
+    "local_group_runs", "append_local_run", "upsample_ocache", "flex_block_mask", "block_mask_to_lists",
+    "key_block_sums", "topk_block_lists", "sink_window_topk_block_mask",
+]
+
+
+def scale_offsets(scales: Sequence[int] = INFINITY_SCALES) -> List[int]:
+    """Start offset of every scale on the concatenated key axis (``cum`` of
+    models/sparvar/sparse_attn.py:908-909): [0, 1, 5, 21, ..., 10521]."""
+    offs = [0]
+    for s in scales:
+        offs.append(offs[-1] + s * s)
+    return offs
+
+
+def indices_count(top_keys: float, k_len: int, multiple_of: Optional[int] = None) -> int:
+    """Number of keys kept per query group: ``m * round(top_keys * Lk / m)``, half-to-even
+    (models/sparvar/sparse_attn.py:1012)."""
+    m = get_kernel_config_attn()["counts_multiple_of"] if multiple_of is None else multiple_of
+    return int(m * round((top_keys * k_len) / m))
+
+
+def topk_index_list(bs: torch.Tensor, top_keys: float, multiple_of: Optional[int] = None,
+                    indices_pad_to: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Full-step list build (models/sparvar/sparse_attn.py:1012-1036): descending top-k of the
+    colsum ``bs`` [B,H,G,Lk] -> ``inds`` int32 [B,H,G,Lk] whose first ``count`` columns are valid,
+    and ``counts`` int32 [B,H,G].  Padding columns are zero-filled (the reference leaves them
+    uninitialised; they are never read)."""
+    cfg = get_kernel_config_attn()
+    m = cfg["counts_multiple_of"] if multiple_of is None else multiple_of
+    B, H, G, Lk = bs.shape
+    cnt = indices_count(top_keys, Lk, m)
+    if cnt > Lk:
+        raise ValueError(f"top-k count {cnt} exceeds key length {Lk}")
+    inds = torch.zeros((B, H, G, Lk), dtype=torch.int32, device=bs.device)
+    if cnt > 0:
+        inds[..., :cnt] = torch.topk(bs, k=cnt, dim=-1).indices.to(torch.int32)
+    counts = torch.full((B, H, G), cnt, dtype=torch.int32, device=bs.device)
+    return inds, counts
+
+
+def map_inds_counts_across_scales(inds_S: torch.Tensor, counts_S, cur_q_len: int, cur_k_len: int,
+                                  bm: int = 192, indices_pad_to: int = 1) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Nearest query-group remap of a key list from the decision scale to the current scale
+    (models/sparvar/sparse_attn.py:366-421, the path without sink).  ``counts_S`` may be a tensor
+    (its [0,0,0] element is read, one host sync as in the reference) or a Python int."""
+    B, H, Gs, Ks = inds_S.shape
+    Gk = (cur_q_len + bm - 1) // bm
+    raw = int(counts_S[0, 0, 0]) if torch.is_tensor(counts_S) else int(counts_S)
+    cnt = max(indices_pad_to, (raw + indices_pad_to - 1) // indices_pad_to * indices_pad_to)
+    centers = torch.arange(Gk, device=inds_S.device, dtype=torch.float32) + 0.5
+    src = torch.round(centers / Gk * Gs - 0.5).to(torch.int64).clamp_(0, Gs - 1)
+    templ = inds_S.index_select(2, src)
+    if Ks >= cnt:
+        out = templ[..., :cnt].to(torch.int32)
+    else:
+        out = templ.repeat_interleave(math.ceil(cnt / Ks), dim=-1)[..., :cnt].to(torch.int32)
+    out = out.clamp(0, max(0, cur_k_len - 1)).contiguous()
+    counts = torch.full((B, H, Gk), cnt, dtype=torch.int32, device=inds_S.device)
+    return out, counts
+
+
+def local_group_runs(scale_idx: int, win: int, bm: int = 192, counts_multiple_of: Optional[int] = None,
+                     scales: Sequence[int] = INFINITY_SCALES, device=None) -> Tuple[torch.Tensor, int]:
+    """Local-window key run of every query group of scale ``scale_idx`` (the composition of
+    ``local_window_indices``, ``build_crossscale_indices`` with ``{0: (win, win)}`` and
+    ``aggregate_group_indices``, models/sparvar/sparse_attn.py:620-674, 678-768, 778-857, as used at
+    :921-938): the union of the clamp-padded win x win windows of the group's queries fixes a
+    first key and a count; the count, rounded up to ``counts_multiple_of`` and maximised over
+    groups, gives ONE contiguous run ``[tail-(L-1), tail]``, ``tail = min(first+L-1, Lk-1)``.
+    Returns (int64 [G, L], L)."""
+    m = get_kernel_config_attn()["counts_multiple_of"] if counts_multiple_of is None else counts_multiple_of
+    offs = scale_offsets(scales)
+    S = scales[scale_idx]
+    base, kv_len, q_len = offs[scale_idx], offs[scale_idx + 1], S * S
+    ry = (win - 1) // 2
+    d = torch.arange(-ry, win - ry, device=device)
+    y = torch.arange(S, device=device)
+    ny = (y[:, None] + d[None, :]).clamp_(0, S - 1)                        # [S, win]
+    lin = (ny[:, None, :, None] * S + ny[None, :, None, :]).reshape(q_len, win * win) + base
+    G = (q_len + bm - 1) // bm
+    firsts, cnts = [], []
+    for g in range(G):
+        u = torch.unique(lin[g * bm:min((g + 1) * bm, q_len)])
+        c = int(u.numel())
+        if m and m > 1:
+            c = (c + m - 1) // m * m
+        firsts.append(int(u[0]))
+        cnts.append(c)
+    run = max(cnts)
+    first = torch.tensor(firsts, device=device, dtype=torch.int64)
+    tail = torch.clamp(first + (run - 1), max=kv_len - 1)
+    out = (tail[:, None] - (run - 1)) + torch.arange(run, device=device, dtype=torch.int64)[None, :]
+    return out, run
+
+
+def append_local_run(inds: torch.Tensor, count: int, local_inds: torch.Tensor, local_count: int, k_len: int,
+                     multiple_of: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Sparse-step list: remapped top-k keys followed by the scale's local run
+    (models/sparvar/sparse_attn.py:1096-1121).  ``inds`` [B,H,G,count], ``local_inds`` [G,local_count]
+    -> (int32 [B,H,G,k_len] zero-padded, counts int32 [B,H,G] = count + local_count)."""
+    m = get_kernel_config_attn()["counts_multiple_of"] if multiple_of is None else multiple_of
+    B, H, G, _ = inds.shape
+    total = count + local_count
+    assert total % m == 0, f"after add local sparse index, mismatch multiple_of={m}"
+    if total > k_len:
+        raise ValueError(f"list length {total} exceeds key length {k_len}")
+    out = torch.zeros((B, H, G, k_len), dtype=torch.int32, device=inds.device)
+    out[..., :count] = inds[..., :count]
+    out[..., count:total] = local_inds.to(device=inds.device, dtype=torch.int32).expand(B, H, G, local_count)
+    counts = torch.full((B, H, G), total, dtype=torch.int32, device=inds.device)
+    return out, counts
+
+
+def upsample_ocache(o_cache: torch.Tensor, L_src: int, L_tgt: int) -> torch.Tensor:
+    """Bilinear (align_corners=False) upsample of an O-cache stored as an h x h token grid
+    (``upsample_Ocache``, models/sparvar/sparse_attn.py:324-362)."""
+    B, H, _, Dh = o_cache.shape
+    hs, ht = int(L_src ** 0.5), int(L_tgt ** 0.5)
+    x = o_cache.view(B, H, hs, hs, Dh).permute(0, 1, 4, 2, 3).reshape(B * H, Dh, hs, hs)
+    x = F.interpolate(x, size=(ht, ht), mode="bilinear", align_corners=False)
+    return x.view(B, H, Dh, ht, ht).permute(0, 1, 3, 4, 2).reshape(B, H, ht * ht, Dh)
+
+
+def flex_block_mask(q_scale_idx: int, kernel_schedule: Sequence[int], attn_sink_scale: int, block_size: int = 128,
+                    block_k: Optional[int] = None, scales: Sequence[int] = INFINITY_SCALES, device=None) -> torch.Tensor:
+    """Attention-sink + local-window block mask of ``SparseFlexAttn``
+    (models/sparvar/basic_sparvar.py:74-185): a key is attended if it lies below
+    ``cum[attn_sink_scale]`` or inside the square window (per-key-scale kernel size, negative =
+    never) around the query position rescaled to the key's grid; a block is kept if any of its
+    elements is.  Returns bool [nQ, nK] for (block_size x block_k) blocks."""
+    bq, bk = block_size, (block_size if block_k is None else block_k)
+    offs = scale_offsets(scales)
+    Hq = scales[q_scale_idx]
+    Sq, Sk = Hq * Hq, offs[q_scale_idx + 1]
+    sink = offs[attn_sink_scale] if attn_sink_scale > 0 else 0
+    kv = torch.arange(Sk, device=device)
+    bounds = torch.tensor(offs[:q_scale_idx + 2], device=device)
+    si = torch.searchsorted(bounds, kv, right=True) - 1
+    Hk = torch.tensor(list(scales[:q_scale_idx + 1]), device=device)[si]
+    ksz = torch.tensor(list(kernel_schedule[:q_scale_idx + 1]), device=device)[si]
+    rel = kv - bounds[si]
+    ky, kx = rel // Hk, rel % Hk
+    qi = torch.arange(Sq, device=device)
+    qy, qx = (qi // Hq).float(), (qi % Hq).float()
+    cy = torch.round((qy / Hq)[:, None] * Hk[None, :])
+    cx = torch.round((qx / Hq)[:, None] * Hk[None, :])
+    half = torch.div(ksz, 2, rounding_mode="floor")[None, :]
+    fine = ((cy - ky[None, :]).abs() <= half) & ((cx - kx[None, :]).abs() <= half)
+    fine |= (kv < sink)[None, :]
+    pq, pk = (-Sq) % bq, (-Sk) % bk
+    fine = F.pad(fine, (0, pk, 0, pq), value=False)
+    return fine.view((Sq + pq) // bq, bq, (Sk + pk) // bk, bk).permute(0, 2, 1, 3).flatten(2).any(-1)
+
+
+def block_mask_to_lists(mask: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bool [..., nQ, nK] -> flex ``BlockMask`` lists: ``kv_num_blocks`` int32 [..., nQ] and
+    ``kv_indices`` int32 [..., nQ, nK] (kept blocks first, ascending; unused tail zero)."""
+    nK = mask.shape[-1]
+    num = mask.sum(-1, dtype=torch.int32)
+    # kept blocks sort before dropped ones, both in ascending block order
+    key = (~mask).to(torch.int32) * nK + torch.arange(nK, device=mask.device, dtype=torch.int32)
+    order = torch.argsort(key, dim=-1).to(torch.int32)
+    keep = torch.arange(nK, device=mask.device) < num.unsqueeze(-1)
+    return num, torch.where(keep, order, torch.zeros_like(order)).contiguous()
+
+
+def key_block_sums(cs: torch.Tensor, block_k: int = 64) -> torch.Tensor:
+    """Sum of a colsum over blocks of ``block_k`` consecutive keys (ragged last block)."""
+    Lk = cs.shape[-1]
+    nb = (Lk + block_k - 1) // block_k
+    return F.pad(cs, (0, nb * block_k - Lk)).unflatten(-1, (nb, block_k)).sum(-1)
+
+
+def topk_block_lists(block_scores: torch.Tensor, keep_ratio: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Top ``round(keep_ratio*nK)`` key blocks per row (at least one), as sorted block lists."""
+    nK = block_scores.shape[-1]
+    k = max(1, min(nK, int(round(keep_ratio * nK))))
+    idx = torch.topk(block_scores, k=k, dim=-1).indices.sort(-1).values.to(torch.int32)
+    num = torch.full(block_scores.shape[:-1], k, dtype=torch.int32, device=block_scores.device)
+    return num, idx.contiguous()
+
+
+def sink_window_topk_block_mask(block_scores: torch.Tensor, block_q: int = 128, block_k: int = 64, density: float = 0.25,
+                                sink_scale: int = 7, window: int = 2, scales: Sequence[int] = INFINITY_SCALES) -> torch.Tensor:
+    """Block mask of the Infinity last-scale benchmark configuration: all key blocks of scales
+    below ``sink_scale`` (keys < 521), +-``window`` key blocks around the query block's position
+    rescaled into every later scale, then the best-scoring remaining blocks by ``block_scores``
+    [B,H,nQ,nK] (colsum summed per query block and key block) up to ``round(density*nK)`` per row."""
+    offs = scale_offsets(scales)
+    Hq = scales[-1]
+    Sq, Sk = Hq * Hq, offs[-1]
+    nQ, nK = (Sq + block_q - 1) // block_q, (Sk + block_k - 1) // block_k
+    dev = block_scores.device
+    assert tuple(block_scores.shape[2:]) == (nQ, nK), (tuple(block_scores.shape), nQ, nK)
+    base = torch.zeros(nQ, nK, dtype=torch.bool, device=dev)
+    base[:, :(offs[sink_scale] + block_k - 1) // block_k] = True
+    qc = torch.clamp(torch.arange(nQ, device=dev) * block_q + block_q // 2, max=Sq - 1)
+    qy, qx = qc // Hq, qc % Hq
+    cols = torch.arange(nK, device=dev)[None, :]
+    for si in range(sink_scale, len(scales)):
+        Hk = scales[si]
+        ky = torch.clamp(qy * Hk // Hq, max=Hk - 1)
+        kx = torch.clamp(qx * Hk // Hq, max=Hk - 1)
+        j = (offs[si] + ky * Hk + kx) // block_k
+        lo = torch.clamp(j - window, min=offs[si] // block_k)[:, None]
+        hi = torch.clamp(j + window, max=(offs[si + 1] - 1) // block_k)[:, None]
+        base |= (cols >= lo) & (cols <= hi)
+    target = int(round(density * nK))
+    extra = (target - base.sum(-1)).clamp(min=0)                               # [nQ]
+    score = block_scores.to(torch.float32).masked_fill(base, -float("inf"))
+    rank = torch.argsort(torch.argsort(score, dim=-1, descending=True, stable=True), dim=-1, stable=True)
+    return base | (rank < extra[None, None, :, None])
