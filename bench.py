@@ -119,6 +119,7 @@ def main():
     ap.add_argument("--workload", default="block_sparse_25",
                     help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | density_<pct> | video_10")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-aux", action="store_true", help="skip the companion dense/colsum/mask-build timings")
     ap.add_argument("--cpu-budget-s", type=float, default=20.0)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -226,7 +227,7 @@ def main():
     ms, wall_ms = time_launches(fn, args.steps, args.warmup)
     tflops = flops / (ms * 1e-3) / 1e12
 
-    if wl == "block_sparse_25":
+    if wl == "block_sparse_25" and not args.no_aux:
         # companion numbers named by the metric: colsum (+ mask build) versus the dense attention it replaces
         dense_ms, _ = time_launches(lambda: ops.dense_attn(qg, kg, vg, scale), 10, 3)
         M, L = ops._lse_only(qg, kg, scale)

@@ -33,11 +33,12 @@ def load() -> C.CDLL:
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    path = os.environ.get("LVAR_AMD_LIB", LIB_PATH)  # override for debug builds of the same ABI
+    if not os.path.exists(path):
         raise ImportError(
-            f"{LIB_PATH} is missing: build it with `python -m lvar_amd.build` (needs hipcc). "
+            f"{path} is missing: build it with `python -m lvar_amd.build` (needs hipcc). "
             "lvar_amd has no CPU or PyTorch fallback.")
-    lib = C.CDLL(LIB_PATH)
+    lib = C.CDLL(path)
     T, P, I, I64, F = LvarTensor, C.c_void_p, C.c_int, C.c_int64, C.c_float
     lib.lvar_version.restype = I
     lib.lvar_version.argtypes = []

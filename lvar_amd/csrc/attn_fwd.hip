@@ -2,19 +2,25 @@
 // (flex BlockMask layout) and token-list (column-sparse, gathered keys) variants.
 //
 // Work decomposition
-//   workgroup  = NWAVES waves, 32 query rows per wave, all waves share one K/V tile in LDS
+//   workgroup  = NWAVES waves, 32 query rows per wave, all waves share the K/V tiles in LDS
 //   wave       = S^T[64 keys x 32 queries] = K_tile . Q^T with 32x32x16 bf16 MFMA (K rows are
 //                the A operand read from LDS, Q^T is the B operand held in registers), so a
 //                lane owns ONE query column: the softmax row max / sum are in-register
 //                reductions plus one exchange with lane^32.
 //                O^T[d x 32 queries] += V^T . P^T: the S^T accumulators, packed to bf16, are
-//                already in B-operand layout; V^T comes from a row-major V tile through
+//                already in B-operand layout; V^T comes from the row-major V tile through
 //                transposing LDS reads (ds_read_b64_tr_b16).
-//   pipeline   = K/V tile t+1 is fetched global->registers while tile t is computed, then
-//                stored to the other LDS stage; one barrier per tile.
+//   data path  = K/V rows go global -> LDS directly (buffer_load ... lds, 16 B per lane, no
+//                register staging).  An instruction fills 1 KiB of consecutive LDS, so rows are
+//                unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte chunk index
+//                applied on the global side (each lane fetches the chunk that belongs in its slot).
+//   pipeline   = iteration t issues the loads of K(t+2) and V(t+1), computes S(t+1) = K(t+1) Q^T on
+//                the matrix cores while the vector ALU runs the softmax of S(t), then O += P(t) V(t);
+//                K and V are double-buffered, one barrier per tile.
 // Softmax runs in the exp2 domain with a lazily updated reference maximum: accumulators are
 // rescaled only when some row maximum grows by more than RESCALE_TAU, which is exact
 // because numerator and denominator share the same reference.
+#include <type_traits>
 #include "common.h"
 #include "launch.h"
 
@@ -23,17 +29,33 @@ namespace lvar {
 static constexpr float RESCALE_TAU = 8.0f;
 static constexpr float NEG_BIG = -1.0e30f;
 
+template <int D>
+struct Swz {
+  static constexpr int ROWB = D * 2;      // bytes per K/V row
+  static constexpr int CPR = ROWB / 16;   // 16-byte chunks per row
+  // chunk-index XOR of the K tile: makes ds_read_b128 of 16 consecutive rows conflict-free
+  __device__ static __forceinline__ int fk(int row) { return (row / (256 / ROWB)) & (CPR - 1); }
+  // chunk-index XOR of the V tile: moves the 64-byte segment read by the transposing loads of
+  // 4 consecutive rows onto 4 different bank groups
+  __device__ static __forceinline__ int fv(int row) { return (D == 128) ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+};
+
 template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY>
 __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_kernel(const AttnParams p) {
-  constexpr int NT = NWAVES * 64, WGROWS = NWAVES * 32;
-  constexpr int KS = D / 16, MTD = D / 32, CPR = D / 8;
-  constexpr int KSTR = D * 2 + 16, VSTR = D * 2 + 64;
-  constexpr int CHUNKS = 64 * CPR, CPT = (CHUNKS + NT - 1) / NT;
-  constexpr bool EXACT = (CHUNKS % NT) == 0;
-  constexpr int STAGE = 64 * (KSTR + VSTR);
+  // The body is compiled for the device only: the host pass just needs the launch stub, and it
+  // silently drops the stub when the body uses the LDS-DMA builtins.
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int WGROWS = NWAVES * 32;
+  constexpr int KS = D / 16, MTD = D / 32;
+  constexpr int ROWB = Swz<D>::ROWB, CPR = Swz<D>::CPR;
+  constexpr int RPI = 1024 / ROWB;          // rows filled by one 64-lane x 16 B load
+  constexpr int NI = 64 / RPI;              // loads per 64-row tile
+  constexpr int SLOTS = (NI + NWAVES - 1) / NWAVES;
+  constexpr int TILE = 64 * ROWB;
   constexpr int OSTR = D * 2 + 16;  // epilogue transpose buffer row stride (bytes)
-  static_assert(NWAVES * 32 * OSTR <= 2 * STAGE, "epilogue buffer must fit in the K/V stages");
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+  static_assert(NWAVES * 32 * OSTR <= 4 * TILE, "epilogue buffer must fit in the K/V buffers");
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  // LDS map: K buffers at 0 and TILE, V buffers at 2*TILE and 3*TILE
 
   // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; remap so that each XCD
   // walks a contiguous range of (batch, head, q-tile) and K/V of one head stay in its L2.
@@ -42,7 +64,8 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   if (w >= p.total_wg) return;
   const int bh = w / p.nqt, qt = w - bh * p.nqt;
   const int b = bh / p.H, h = bh - b * p.H;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, r = lane & 31;
   const int q0 = qt * WGROWS;
   const int g = q0 / p.group_rows;
@@ -57,64 +80,6 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     T = (MODE == MODE_BLOCK) ? (count << p.sub_shift) : ((count + 63) >> 6);
   }
 
-  const bf16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
-  const bf16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
-
-  // per-thread chunk coordinates inside a tile
-  int crow[CPT], ccol[CPT];
-#pragma unroll
-  for (int i = 0; i < CPT; i++) {
-    int c = tid + i * NT;
-    crow[i] = c / CPR;
-    ccol[i] = c - crow[i] * CPR;
-  }
-
-  auto fetch_rows = [&](int t, int (&rows)[CPT], int& nvalid) {
-    if (MODE == MODE_DENSE) {
-      int base = t << 6;
-      nvalid = min(64, p.Lk - base);
-#pragma unroll
-      for (int i = 0; i < CPT; i++) rows[i] = min(base + crow[i], p.Lk - 1);
-    } else if (MODE == MODE_BLOCK) {
-      int blk = list[t >> p.sub_shift];
-      int base = ((blk << p.sub_shift) + (t & ((1 << p.sub_shift) - 1))) << 6;
-      nvalid = max(0, min(64, p.Lk - base));
-#pragma unroll
-      for (int i = 0; i < CPT; i++) rows[i] = max(0, min(base + crow[i], p.Lk - 1));
-    } else {
-      int base = t << 6;
-      nvalid = min(64, count - base);
-#pragma unroll
-      for (int i = 0; i < CPT; i++) {
-        int pos = base + crow[i];
-        int idx = (pos < count && (EXACT || crow[i] < 64)) ? list[pos] : 0;
-        rows[i] = max(0, min(idx, p.Lk - 1));
-      }
-    }
-  };
-
-  u32x4 kreg[CPT], vreg[CPT];
-  auto load_tile = [&](const int (&rows)[CPT]) {
-#pragma unroll
-    for (int i = 0; i < CPT; i++) {
-      if (EXACT || tid + i * NT < CHUNKS) {
-        kreg[i] = *(const u32x4*)(kbase + (int64_t)rows[i] * p.k_sr + ccol[i] * 8);
-        if (!LSE_ONLY) vreg[i] = *(const u32x4*)(vbase + (int64_t)rows[i] * p.v_sr + ccol[i] * 8);
-      }
-    }
-  };
-  auto store_tile = [&](int stage) {
-    char* ks = smem + stage * STAGE;
-    char* vs = ks + 64 * KSTR;
-#pragma unroll
-    for (int i = 0; i < CPT; i++) {
-      if (EXACT || tid + i * NT < CHUNKS) {
-        *(u32x4*)(ks + crow[i] * KSTR + ccol[i] * 16) = kreg[i];
-        if (!LSE_ONLY) *(u32x4*)(vs + crow[i] * VSTR + ccol[i] * 16) = vreg[i];
-      }
-    }
-  };
-
   // accumulators and softmax state (one query column per lane pair l, l^32)
   f32x16 oacc[MTD];
 #pragma unroll
@@ -125,6 +90,49 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const float c = p.c;
 
   if (T > 0) {
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(p.k + b * p.k_sb + h * p.k_sh), 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(p.v + b * p.v_sb + h * p.v_sh), 0, 0x7fffffff, 0x00020000);
+    const int k_srb = (int)p.k_sr * 2, v_srb = (int)p.v_sr * 2;  // row strides in bytes
+
+    // per-lane role in a tile load: row (within the RPI rows of one instruction) and chunk slot
+    const int lrow = lane / CPR, lcs = lane % CPR;
+
+    // Rows (in the K/V tensors, clamped into [0, Lk)) that this lane fetches for tile t, one per
+    // load slot, and nvalid = number of leading tile rows that take part in the softmax.
+    auto fetch_rows = [&](int t, int (&rows)[SLOTS], int& nvalid) {
+      int base;
+      if (MODE == MODE_BLOCK) {
+        const int blk = list[t >> p.sub_shift];
+        base = ((blk << p.sub_shift) + (t & ((1 << p.sub_shift) - 1))) << 6;
+        nvalid = max(0, min(64, p.Lk - base));
+      } else {
+        base = t << 6;
+        nvalid = min(64, (MODE == MODE_DENSE ? p.Lk : count) - base);
+      }
+#pragma unroll
+      for (int s = 0; s < SLOTS; s++) {
+        const int trow = (wave + s * NWAVES) * RPI + lrow;
+        int grow = base + trow;
+        if (MODE == MODE_GATHER) grow = (grow < count && trow < 64) ? list[grow] : 0;
+        rows[s] = max(0, min(grow, p.Lk - 1));
+      }
+    };
+    // issue the global->LDS loads of one tile (K or V) into LDS buffer `dst`
+    auto issue = [&](const __amdgpu_buffer_rsrc_t& rsrc, int srb, bool is_v, const int (&rows)[SLOTS], char* dst) {
+#pragma unroll
+      for (int s = 0; s < SLOTS; s++) {
+        const int i = wave + s * NWAVES;
+        if ((NI % NWAVES == 0) || i < NI) {
+          const int trow = i * RPI + lrow;
+          const int chunk = lcs ^ (is_v ? Swz<D>::fv(trow) : Swz<D>::fk(trow));
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (LVAR_LDS void*)(dst + i * 1024), 16,
+                                                   rows[s] * srb + chunk * 16, 0, 0, 0);
+        }
+      }
+    };
+
     // Q^T fragments stay in registers for the whole key loop
     const int qrow = min(q0 + wave * 32 + r, p.Lq - 1);
     const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qrow * p.q_sr + hh * 8;
@@ -132,43 +140,33 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qf[ks] = *(const bf16x8*)(qp + ks * 16);
 
-    int rows_next[CPT], nv_cur, nv_next = 0;
-    {
-      int rows0[CPT];
-      fetch_rows(0, rows0, nv_cur);
-      load_tile(rows0);
-      if (T > 1) fetch_rows(1, rows_next, nv_next);
-      store_tile(0);
-    }
-    __syncthreads();
+    // per-lane LDS read offsets (swizzled); K: row r (+32), chunk 2*ks+hh; V: see lds_read_tr
+    const int kbase_l = r * ROWB + ((hh ^ Swz<D>::fk(r)) << 4);
+    const int sq = (lane & 15) >> 2, sm = lane & 3;
+    const int vbase_l = (4 * hh + sq) * ROWB + (((Swz<D>::fv(sq)) | (((lane >> 4) & 1) << 1) | (sm >> 1)) << 4) + (sm & 1) * 8;
 
-    for (int t = 0; t < T; t++) {
-      const int stage = t & 1;
-      if (t + 1 < T) load_tile(rows_next);
-      int nv_next2 = 0;
-      if (t + 2 < T) fetch_rows(t + 2, rows_next, nv_next2);
-
-      // ---- S^T = K_tile . Q^T ----
-      f32x16 s0, s1;
+    auto qk_tile = [&](const char* kbuf, f32x16& s0, f32x16& s1) {
 #pragma unroll
       for (int i = 0; i < 16; i++) { s0[i] = 0.f; s1[i] = 0.f; }
-      const char* kl = smem + stage * STAGE + r * KSTR + hh * 16;
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
-        bf16x8 a0 = *(const bf16x8*)(kl + ks * 32);
-        bf16x8 a1 = *(const bf16x8*)(kl + 32 * KSTR + ks * 32);
+        const char* a = kbuf + (kbase_l ^ (ks << 5));
+        bf16x8 a0 = *(const bf16x8*)(a);
+        bf16x8 a1 = *(const bf16x8*)(a + 32 * ROWB);
         s0 = mfma32(a0, qf[ks], s0);
         s1 = mfma32(a1, qf[ks], s1);
       }
-      if (nv_cur < 64) {
+    };
+
+    auto softmax_pv = [&](f32x16& s0, f32x16& s1, int nvalid, const char* vbuf) {
+      if (nvalid < 64) {
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          int kr = 8 * (i >> 2) + 4 * hh + (i & 3);
-          if (kr >= nv_cur) s0[i] = -INFINITY;
-          if (kr + 32 >= nv_cur) s1[i] = -INFINITY;
+          const int kr = 8 * (i >> 2) + 4 * hh + (i & 3);
+          if (kr >= nvalid) s0[i] = -INFINITY;
+          if (kr + 32 >= nvalid) s1[i] = -INFINITY;
         }
       }
-      // ---- online softmax (base 2) ----
       float mx = fmaxf(s0[0], s1[0]);
 #pragma unroll
       for (int i = 1; i < 16; i++) mx = fmaxf(mx, fmaxf(s0[i], s1[i]));
@@ -195,29 +193,64 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
         lsum += s0[i] + s1[i];
       }
       if (!LSE_ONLY) {
-        // ---- O^T += V^T . P^T ----
         bf16x8 pb[4];
         pb[0] = pack8(s0[0], s0[1], s0[2], s0[3], s0[4], s0[5], s0[6], s0[7]);
         pb[1] = pack8(s0[8], s0[9], s0[10], s0[11], s0[12], s0[13], s0[14], s0[15]);
         pb[2] = pack8(s1[0], s1[1], s1[2], s1[3], s1[4], s1[5], s1[6], s1[7]);
         pb[3] = pack8(s1[8], s1[9], s1[10], s1[11], s1[12], s1[13], s1[14], s1[15]);
-        const char* vl = smem + stage * STAGE + 64 * KSTR + (((lane & 15) >> 2) + 4 * hh) * VSTR +
-                         ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
 #pragma unroll
         for (int kb = 0; kb < 4; kb++) {
 #pragma unroll
           for (int m = 0; m < MTD; m++) {
-            bf16x4 lo = lds_read_tr(vl + (kb * 16) * VSTR + m * 64);
-            bf16x4 hi = lds_read_tr(vl + (kb * 16 + 8) * VSTR + m * 64);
-            bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            oacc[m] = mfma32(a, pb[kb], oacc[m]);
+            const char* a = vbuf + (vbase_l ^ (m << 6)) + kb * 16 * ROWB;
+            bf16x4 lo = lds_read_tr(a);
+            bf16x4 hi = lds_read_tr(a + 8 * ROWB);
+            bf16x8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            oacc[m] = mfma32(av, pb[kb], oacc[m]);
           }
         }
       }
-      if (t + 1 < T) store_tile(stage ^ 1);
-      nv_cur = nv_next;
-      nv_next = nv_next2;
+    };
+
+    // ---- prologue: tiles 0 and 1 in flight, S(0) computed ----
+    // rows_v: rows of tile t+1 (its V is fetched next), rows_k: rows of tile t+2 (its K is next)
+    int rows_v[SLOTS], rows_k[SLOTS], rows_n[SLOTS];
+    int nv0, nv1 = 0, nv2 = 0, nv3 = 0;
+    fetch_rows(0, rows_n, nv0);
+    if (T > 1) fetch_rows(1, rows_v, nv1);
+    if (T > 2) fetch_rows(2, rows_k, nv2);
+    issue(krsrc, k_srb, false, rows_n, smem);
+    if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows_n, smem + 2 * TILE);
+    if (T > 1) issue(krsrc, k_srb, false, rows_v, smem + TILE);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's LDS fills have landed
+    __syncthreads();
+    f32x16 sa0, sa1, sb0, sb1;
+    qk_tile(smem, sa0, sa1);
+
+    // One iteration; PAR = t & 1 selects the buffers at compile time:
+    //   K(t+1) is in K buffer (1-PAR), K(t+2) goes to K buffer PAR,
+    //   V(t) is in V buffer PAR, V(t+1) goes to V buffer (1-PAR).
+    auto iteration = [&](int t, auto par, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1) {
+      constexpr int PAR = decltype(par)::value;
+      char* kb_cur = smem + PAR * TILE;
+      char* kb_nxt = smem + (1 - PAR) * TILE;
+      char* vb_cur = smem + (2 + PAR) * TILE;
+      char* vb_nxt = smem + (3 - PAR) * TILE;
+      if (!LSE_ONLY && t + 1 < T) issue(vrsrc, v_srb, true, rows_v, vb_nxt);
+      if (t + 2 < T) issue(krsrc, k_srb, false, rows_k, kb_cur);
+      if (t + 3 < T) fetch_rows(t + 3, rows_n, nv3);
+      if (t + 1 < T) qk_tile(kb_nxt, n0, n1);
+      softmax_pv(c0, c1, nv0, vb_cur);
+      __builtin_amdgcn_s_waitcnt(0x0f70);
       __syncthreads();
+      nv0 = nv1; nv1 = nv2; nv2 = nv3;
+#pragma unroll
+      for (int s = 0; s < SLOTS; s++) { rows_v[s] = rows_k[s]; rows_k[s] = rows_n[s]; }
+    };
+
+    for (int t = 0; t < T; t += 2) {
+      iteration(t, std::integral_constant<int, 0>{}, sa0, sa1, sb0, sb1);
+      if (t + 1 < T) iteration(t + 1, std::integral_constant<int, 1>{}, sb0, sb1, sa0, sa1);
     }
   }
 
@@ -259,23 +292,25 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
   __builtin_amdgcn_wave_barrier();
   bf16_t* op = p.o + b * p.o_sb + h * p.o_sh;
+  constexpr int OCPR = D / 8;
 #pragma unroll
-  for (int i = 0; i < (32 * CPR) / 64; i++) {
+  for (int i = 0; i < (32 * OCPR) / 64; i++) {
     const int cidx = lane + i * 64;
-    const int orow = cidx / CPR, ocol = cidx - orow * CPR;
+    const int orow = cidx / OCPR, ocol = cidx - orow * OCPR;
     const int grow = q0 + wave * 32 + orow;
     if (grow < p.Lq) {
       u32x4 val = *(const u32x4*)(ob + orow * OSTR + ocol * 16);
       *(u32x4*)(op + (int64_t)grow * p.o_sr + ocol * 8) = val;
     }
   }
+#endif  // __HIP_DEVICE_COMPILE__
 }
 
 template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY>
 static int launch_one(const AttnParams& p0, hipStream_t stream) {
   AttnParams p = p0;
   constexpr int WGROWS = NWAVES * 32;
-  constexpr int STAGE = 64 * ((D * 2 + 16) + (D * 2 + 64));
+  constexpr int SMEM = 4 * 64 * D * 2;
   if (p.group_rows % WGROWS != 0 && MODE != MODE_DENSE) return LVAR_EINVAL;
   if (MODE == MODE_DENSE) p.group_rows = WGROWS;
   p.nqt = (p.Lq + WGROWS - 1) / WGROWS;
@@ -283,13 +318,12 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
   const int grid = ((p.total_wg + 7) / 8) * 8;
   auto kern = attn_fwd_kernel<D, NWAVES, MODE, ACCUM, LSE_ONLY>;
   static bool attr_set = false;
-  const int smem = 2 * STAGE;
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != hipSuccess)
       return LVAR_ELAUNCH;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(NWAVES * 64), smem, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(NWAVES * 64), SMEM, stream, p);
   return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
 }
 

@@ -18,6 +18,11 @@ bool view_ok(const lvar_tensor_t& t) {
   return t.ptr && aligned16(t.ptr) && t.stride_b % 8 == 0 && t.stride_h % 8 == 0 && t.stride_row % 8 == 0;
 }
 
+// K/V rows are addressed with 32-bit byte offsets inside one (batch, head) slice
+bool kv_span_ok(const lvar_tensor_t& t, int Lk, int head_dim) {
+  return t.stride_row > 0 && (double)t.stride_row * 2.0 * Lk + head_dim * 2.0 < 2147483647.0;
+}
+
 bool shape_ok(int B, int H, int Lq, int Lk, float scale) {
   return B > 0 && H > 0 && Lq > 0 && Lk > 0 && std::isfinite(scale) && scale > 0.f;
 }
@@ -58,6 +63,7 @@ int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_
                         int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k)) return LVAR_EINVAL;
   const bool lse_only = (o.ptr == nullptr);
+  if (!kv_span_ok(k, Lk, head_dim) || (!lse_only && !kv_span_ok(v, Lk, head_dim))) return LVAR_EINVAL;
   if (!lse_only && (!view_ok(v) || !view_ok(o))) return LVAR_EINVAL;
   if (lse_only && !(M && L)) return LVAR_EINVAL;
   AttnParams p{};
@@ -90,6 +96,7 @@ int lvar_csp_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_te
                       float o_scale, float scale, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
   if (o_accum.ptr && !view_ok(o_accum)) return LVAR_EINVAL;
+  if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
   if (!indices || !counts || G <= 0 || idx_row_stride <= 0) return LVAR_EINVAL;
   if (group_rows <= 0 || group_rows % 32 != 0 || (int64_t)G * group_rows < Lq) return LVAR_EINVAL;
   AttnParams p{};
@@ -118,6 +125,7 @@ int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
                                int64_t stride_ki_q, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
                                int head_dim, float scale, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
+  if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
   if (!kv_num_blocks || !kv_indices || nk_max <= 0) return LVAR_EINVAL;
   if (block_q != 128 || (block_k != 64 && block_k != 128)) return LVAR_EUNSUPPORTED;
   AttnParams p{};
