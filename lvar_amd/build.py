@@ -20,7 +20,8 @@ LIB_PATH = os.path.join(HERE, LIB_NAME)
 SOURCES = ["attn_fwd.hip", "colsum.hip", "capi.hip"]
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off: hipcc must not form v_pk_{add,mul,fma}_f32 from float code
-HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
+# -fno-honor-nans -mno-amdgpu-ieee: max/min map to single v_max/v_max3 without NaN-quieting copies
+HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-fno-honor-nans", "-mno-amdgpu-ieee",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 

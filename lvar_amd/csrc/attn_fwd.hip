@@ -14,9 +14,10 @@
 //                register staging).  An instruction fills 1 KiB of consecutive LDS, so rows are
 //                unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte chunk index
 //                applied on the global side (each lane fetches the chunk that belongs in its slot).
-//   pipeline   = iteration t issues the loads of K(t+2) and V(t+1), computes S(t+1) = K(t+1) Q^T on
-//                the matrix cores while the vector ALU runs the softmax of S(t), then O += P(t) V(t);
-//                K and V are double-buffered, one barrier per tile.
+//   pipeline   = iteration t issues the loads of K(t+2) and V(t+1); the matrix cores run
+//                S(t+1) = K(t+1) Q^T and then O += P(t) V(t) while the vector ALU computes
+//                P(t) = exp2(S(t)) and then the row maximum of S(t+1).  K and V are double-buffered,
+//                one barrier per tile.
 // Softmax runs in the exp2 domain with a lazily updated reference maximum: accumulators are
 // rescaled only when some row maximum grows by more than RESCALE_TAU, which is exact
 // because numerator and denominator share the same reference.
@@ -70,15 +71,20 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const int q0 = qt * WGROWS;
   const int g = q0 / p.group_rows;
 
+  // Key-tile list of this query group.  Dense attention is the block-list variant with a null
+  // list pointer, read as the identity list of ceil(Lk/64) 64-key blocks.
+  const bool identity = (MODE == MODE_BLOCK) && p.list == nullptr;
   const int32_t* list = nullptr;
-  int T, count = 0;
-  if (MODE == MODE_DENSE) {
-    T = (p.Lk + 63) >> 6;
+  int T, count;
+  if (identity) {
+    count = (p.Lk + 63) >> 6;
+    T = count;
   } else {
     count = max(0, min(p.cnt[b * p.cnt_sb + h * p.cnt_sh + g], p.list_len));
     list = p.list + b * p.list_sb + h * p.list_sh + (int64_t)g * p.list_sg;
     T = (MODE == MODE_BLOCK) ? (count << p.sub_shift) : ((count + 63) >> 6);
   }
+  const int sub_shift = identity ? 0 : p.sub_shift;
 
   // accumulators and softmax state (one query column per lane pair l, l^32)
   f32x16 oacc[MTD];
@@ -90,45 +96,70 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const float c = p.c;
 
   if (T > 0) {
-    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(p.k + b * p.k_sb + h * p.k_sh), 0, 0x7fffffff, 0x00020000);
-    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(p.v + b * p.v_sb + h * p.v_sh), 0, 0x7fffffff, 0x00020000);
+    // raw buffer descriptors of this (batch, head) slice of K and V: base, stride 0, no bound
+    auto make_rsrc = [](const void* base) -> i32x4 {
+      const uint64_t a = (uint64_t)base;
+      i32x4 rs = {__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
+                  __builtin_amdgcn_readfirstlane((int)(uint32_t)((a >> 32) & 0xffffu)), 0x7fffffff, 0x00020000};
+      return rs;
+    };
+    const i32x4 krsrc = make_rsrc(p.k + b * p.k_sb + h * p.k_sh);
+    const i32x4 vrsrc = make_rsrc(p.v + b * p.v_sb + h * p.v_sh);
     const int k_srb = (int)p.k_sr * 2, v_srb = (int)p.v_sr * 2;  // row strides in bytes
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(LVAR_LDS char*)smem;
 
     // per-lane role in a tile load: row (within the RPI rows of one instruction) and chunk slot
     const int lrow = lane / CPR, lcs = lane % CPR;
 
-    // Rows (in the K/V tensors, clamped into [0, Lk)) that this lane fetches for tile t, one per
-    // load slot, and nvalid = number of leading tile rows that take part in the softmax.
-    auto fetch_rows = [&](int t, int (&rows)[SLOTS], int& nvalid) {
-      int base;
+    // Tile addressing is a two-step pipeline so that no list load is consumed in the iteration
+    // that issued it: prefetch_raw(t) issues the list reads of tile t, finish_rows(t) turns them
+    // (one iteration later) into a tile descriptor: for token lists the NR = SLOTS rows this lane
+    // fetches, otherwise (NR = 1) the wave-uniform first row of the tile; plus nvalid = number of
+    // leading tile rows that take part in the softmax.
+    constexpr int NR = (MODE == MODE_GATHER) ? SLOTS : 1;
+    auto prefetch_raw = [&](int t, int (&raw)[NR]) {
       if (MODE == MODE_BLOCK) {
-        const int blk = list[t >> p.sub_shift];
-        base = ((blk << p.sub_shift) + (t & ((1 << p.sub_shift) - 1))) << 6;
-        nvalid = max(0, min(64, p.Lk - base));
+        raw[0] = identity ? t : list[t >> sub_shift];
       } else {
-        base = t << 6;
-        nvalid = min(64, (MODE == MODE_DENSE ? p.Lk : count) - base);
-      }
 #pragma unroll
-      for (int s = 0; s < SLOTS; s++) {
-        const int trow = (wave + s * NWAVES) * RPI + lrow;
-        int grow = base + trow;
-        if (MODE == MODE_GATHER) grow = (grow < count && trow < 64) ? list[grow] : 0;
-        rows[s] = max(0, min(grow, p.Lk - 1));
+        for (int s = 0; s < SLOTS; s++) {
+          const int trow = (wave + s * NWAVES) * RPI + lrow;
+          const int pos = (t << 6) + trow;
+          raw[s] = (pos < count && trow < 64) ? list[pos] : 0;
+        }
       }
     };
-    // issue the global->LDS loads of one tile (K or V) into LDS buffer `dst`
-    auto issue = [&](const __amdgpu_buffer_rsrc_t& rsrc, int srb, bool is_v, const int (&rows)[SLOTS], char* dst) {
+    auto finish_rows = [&](int t, const int (&raw)[NR], int (&rows)[NR], int& nvalid) {
+      if (MODE == MODE_BLOCK) {
+        const int blk = __builtin_amdgcn_readfirstlane(raw[0]);
+        rows[0] = ((blk << sub_shift) + (t & ((1 << sub_shift) - 1))) << 6;
+        nvalid = max(0, min(64, p.Lk - rows[0]));
+      } else {
+        nvalid = min(64, count - (t << 6));
+#pragma unroll
+        for (int s = 0; s < NR; s++) rows[s] = raw[s];
+      }
+    };
+    // Issue the global->LDS loads of one tile (K or V) into the LDS buffer at byte address `dst`.
+    // Written as inline assembly so that the compiler does not serialise later LDS reads of the
+    // OTHER buffers behind these fills; completion is awaited with vmcnt(0) before the barrier.
+    auto issue = [&](const i32x4& rsrc, int srb, bool is_v, const int (&rows)[NR], uint32_t dst) {
 #pragma unroll
       for (int s = 0; s < SLOTS; s++) {
         const int i = wave + s * NWAVES;
         if ((NI % NWAVES == 0) || i < NI) {
           const int trow = i * RPI + lrow;
           const int chunk = lcs ^ (is_v ? Swz<D>::fv(trow) : Swz<D>::fk(trow));
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (LVAR_LDS void*)(dst + i * 1024), 16,
-                                                   rows[s] * srb + chunk * 16, 0, 0, 0);
+          const int grow = max(0, min((MODE == MODE_GATHER) ? rows[s < NR ? s : 0] : rows[0] + trow, p.Lk - 1));
+          const int voff = grow * srb + chunk * 16;
+          const uint32_t m0v = dst + i * 1024;
+          asm volatile(
+              "s_mov_b32 m0, %0\n\t"
+              "s_nop 0\n\t"
+              "buffer_load_dwordx4 %1, %2, 0 offen lds"
+              :
+              : "s"(m0v), "v"(voff), "s"(rsrc)
+              : "memory");  // m0 is scratch here: nothing else in this kernel keeps a value in it
         }
       }
     };
@@ -145,6 +176,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     const int sq = (lane & 15) >> 2, sm = lane & 3;
     const int vbase_l = (4 * hh + sq) * ROWB + (((Swz<D>::fv(sq)) | (((lane >> 4) & 1) << 1) | (sm >> 1)) << 4) + (sm & 1) * 8;
 
+    // S^T tile = K_tile . Q^T (16 MFMA for d = 128)
     auto qk_tile = [&](const char* kbuf, f32x16& s0, f32x16& s1) {
 #pragma unroll
       for (int i = 0; i < 16; i++) { s0[i] = 0.f; s1[i] = 0.f; }
@@ -157,20 +189,30 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
         s1 = mfma32(a1, qf[ks], s1);
       }
     };
-
-    auto softmax_pv = [&](f32x16& s0, f32x16& s1, int nvalid, const char* vbuf) {
-      if (nvalid < 64) {
+    // keys beyond nvalid do not take part (only the last tile of a list can be ragged)
+    auto mask_tile = [&](f32x16& s0, f32x16& s1, int nvalid) {
+      // accumulator i of this lane is tile row 8*(i/4) + 4*hh + (i%4): compare against a per-lane
+      // limit so that the per-element constants stay immediates
+      const int lim = nvalid - 4 * hh;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const int kr = 8 * (i >> 2) + 4 * hh + (i & 3);
-          if (kr >= nvalid) s0[i] = -INFINITY;
-          if (kr + 32 >= nvalid) s1[i] = -INFINITY;
-        }
+      for (int i = 0; i < 16; i++) {
+        const int kc = 8 * (i >> 2) + (i & 3);
+        s0[i] = (kc < lim) ? s0[i] : -INFINITY;
+        s1[i] = (kc + 32 < lim) ? s1[i] : -INFINITY;
       }
-      float mx = fmaxf(s0[0], s1[0]);
+    };
+    // row maximum of the raw logits of one tile (both lane halves)
+    auto max_tile = [&](const f32x16& s0, const f32x16& s1) -> float {
+      float ma = fmaxf(s0[0], s1[0]), mb = fmaxf(s0[1], s1[1]);
 #pragma unroll
-      for (int i = 1; i < 16; i++) mx = fmaxf(mx, fmaxf(s0[i], s1[i]));
-      mx = xhalf_max(mx);
+      for (int i = 2; i < 16; i += 2) {
+        ma = fmaxf(fmaxf(ma, s0[i]), s1[i]);
+        mb = fmaxf(fmaxf(mb, s0[i + 1]), s1[i + 1]);
+      }
+      return xhalf_max(fmaxf(ma, mb));
+    };
+    // lazy reference-maximum update for a tile whose raw row maximum is mx
+    auto rescale_check = [&](float mx) {
       const float mt = mx * c;
       m_true = fmaxf(m_true, mt);
       if (__builtin_amdgcn_ballot_w64(mt > m_ref + RESCALE_TAU) != 0) {
@@ -185,72 +227,189 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
         }
         m_ref = m_new;
       }
+    };
+    // P = exp2(S*c - m_ref), row-sum partials, bf16 pack into the B-operand layout of the PV MFMA
+    auto exp_tile = [&](f32x16& s0, f32x16& s1, bf16x8 (&pb)[4]) {
       const float negm = -m_ref;
+      float la = 0.f, lb = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         s0[i] = fast_exp2(fmaf(s0[i], c, negm));
         s1[i] = fast_exp2(fmaf(s1[i], c, negm));
-        lsum += s0[i] + s1[i];
+        la += s0[i];
+        lb += s1[i];
       }
-      if (!LSE_ONLY) {
-        bf16x8 pb[4];
-        pb[0] = pack8(s0[0], s0[1], s0[2], s0[3], s0[4], s0[5], s0[6], s0[7]);
-        pb[1] = pack8(s0[8], s0[9], s0[10], s0[11], s0[12], s0[13], s0[14], s0[15]);
-        pb[2] = pack8(s1[0], s1[1], s1[2], s1[3], s1[4], s1[5], s1[6], s1[7]);
-        pb[3] = pack8(s1[8], s1[9], s1[10], s1[11], s1[12], s1[13], s1[14], s1[15]);
+      lsum += la + lb;
+      pb[0] = pack8(s0[0], s0[1], s0[2], s0[3], s0[4], s0[5], s0[6], s0[7]);
+      pb[1] = pack8(s0[8], s0[9], s0[10], s0[11], s0[12], s0[13], s0[14], s0[15]);
+      pb[2] = pack8(s1[0], s1[1], s1[2], s1[3], s1[4], s1[5], s1[6], s1[7]);
+      pb[3] = pack8(s1[8], s1[9], s1[10], s1[11], s1[12], s1[13], s1[14], s1[15]);
+    };
+    // O^T += V^T . P^T (16 MFMA for d = 128)
+    auto pv_tile = [&](const bf16x8 (&pb)[4], const char* vbuf) {
 #pragma unroll
-        for (int kb = 0; kb < 4; kb++) {
+      for (int kb = 0; kb < 4; kb++) {
 #pragma unroll
-          for (int m = 0; m < MTD; m++) {
-            const char* a = vbuf + (vbase_l ^ (m << 6)) + kb * 16 * ROWB;
-            bf16x4 lo = lds_read_tr(a);
-            bf16x4 hi = lds_read_tr(a + 8 * ROWB);
-            bf16x8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            oacc[m] = mfma32(av, pb[kb], oacc[m]);
-          }
+        for (int m = 0; m < MTD; m++) {
+          const char* a = vbuf + (vbase_l ^ (m << 6)) + kb * 16 * ROWB;
+          bf16x4 lo = lds_read_tr(a);
+          bf16x4 hi = lds_read_tr(a + 8 * ROWB);
+          bf16x8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          oacc[m] = mfma32(av, pb[kb], oacc[m]);
         }
       }
     };
 
     // ---- prologue: tiles 0 and 1 in flight, S(0) computed ----
-    // rows_v: rows of tile t+1 (its V is fetched next), rows_k: rows of tile t+2 (its K is next)
-    int rows_v[SLOTS], rows_k[SLOTS], rows_n[SLOTS];
-    int nv0, nv1 = 0, nv2 = 0, nv3 = 0;
-    fetch_rows(0, rows_n, nv0);
-    if (T > 1) fetch_rows(1, rows_v, nv1);
-    if (T > 2) fetch_rows(2, rows_k, nv2);
-    issue(krsrc, k_srb, false, rows_n, smem);
-    if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows_n, smem + 2 * TILE);
-    if (T > 1) issue(krsrc, k_srb, false, rows_v, smem + TILE);
+    // rows_v: rows of tile t+1 (its V is fetched next), rows_k: rows of tile t+2 (its K is next),
+    // rows_n: rows of tile t+3, raw: list reads of tile t+4
+    int rows_v[NR], rows_k[NR], rows_n[NR], raw[NR];
+#pragma unroll
+    for (int s = 0; s < NR; s++) { rows_v[s] = 0; rows_k[s] = 0; rows_n[s] = 0; raw[s] = 0; }
+    int nv0, nv1 = 64, nv2 = 64, nv3 = 64;
+    {
+      int rows0[NR];
+      prefetch_raw(0, raw);
+      finish_rows(0, raw, rows0, nv0);
+      if (T > 1) { prefetch_raw(1, raw); finish_rows(1, raw, rows_v, nv1); }
+      if (T > 2) { prefetch_raw(2, raw); finish_rows(2, raw, rows_k, nv2); }
+      if (T > 3) prefetch_raw(3, raw);
+      issue(krsrc, k_srb, false, rows0, lds0);
+      if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows0, lds0 + 2 * TILE);
+      if (T > 1) issue(krsrc, k_srb, false, rows_v, lds0 + TILE);
+    }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's LDS fills have landed
     __syncthreads();
     f32x16 sa0, sa1, sb0, sb1;
     qk_tile(smem, sa0, sa1);
+    if (nv0 < 64) mask_tile(sa0, sa1, nv0);
+    rescale_check(max_tile(sa0, sa1));
 
-    // One iteration; PAR = t & 1 selects the buffers at compile time:
+    // Pipelined iteration for a tile t that has a successor; PAR = t & 1 picks the buffers:
     //   K(t+1) is in K buffer (1-PAR), K(t+2) goes to K buffer PAR,
     //   V(t) is in V buffer PAR, V(t+1) goes to V buffer (1-PAR).
-    auto iteration = [&](int t, auto par, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1) {
+    // Between the two barriers the body is one straight-line block: the matrix cores run
+    // S(t+1) = K(t+1) Q^T and then O += P(t) V(t) while the vector ALU turns S(t) into P(t) and
+    // then reduces the row maximum of S(t+1); the reference-maximum update (a rare branch)
+    // sits after the barrier.
+    auto body = [&](int t, auto par, auto masked, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1) {
       constexpr int PAR = decltype(par)::value;
-      char* kb_cur = smem + PAR * TILE;
-      char* kb_nxt = smem + (1 - PAR) * TILE;
-      char* vb_cur = smem + (2 + PAR) * TILE;
-      char* vb_nxt = smem + (3 - PAR) * TILE;
-      if (!LSE_ONLY && t + 1 < T) issue(vrsrc, v_srb, true, rows_v, vb_nxt);
-      if (t + 2 < T) issue(krsrc, k_srb, false, rows_k, kb_cur);
-      if (t + 3 < T) fetch_rows(t + 3, rows_n, nv3);
-      if (t + 1 < T) qk_tile(kb_nxt, n0, n1);
-      softmax_pv(c0, c1, nv0, vb_cur);
+      constexpr bool MASKED = decltype(masked)::value;
+      if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows_v, lds0 + (3 - PAR) * TILE);
+      if (t + 2 < T) issue(krsrc, k_srb, false, rows_k, lds0 + PAR * TILE);
+      if (t + 3 < T) finish_rows(t + 3, raw, rows_n, nv3);
+      if (t + 4 < T) prefetch_raw(t + 4, raw);
+      // The block below is software-pipelined by hand; sched_barrier(0) after every step stops the
+      // compiler from regrouping it.  Phase A: QK MFMA j | K-fragment read j+4 | exp2 of two
+      // elements of S(t).  Phase B: PV MFMA j | the two transposing V reads of MFMA j+4 | a slice
+      // of the row-maximum reduction of S(t+1).
+      constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = 4;
+      const char* kbuf = smem + (1 - PAR) * TILE;
+      const char* vbuf = smem + (2 + PAR) * TILE;
+      auto kread = [&](int j) -> bf16x8 {
+        return *(const bf16x8*)(kbuf + (kbase_l ^ ((j >> 1) << 5)) + (j & 1) * 32 * ROWB);
+      };
+      auto vread = [&](int j) -> bf16x8 {
+        const int kb = j / MTD, m = j % MTD;
+        const char* a = vbuf + (vbase_l ^ (m << 6)) + kb * 16 * ROWB;
+        bf16x4 lo = lds_read_tr(a);
+        bf16x4 hi = lds_read_tr(a + 8 * ROWB);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      };
+#pragma unroll
+      for (int i = 0; i < 16; i++) { n0[i] = 0.f; n1[i] = 0.f; }
+      bf16x8 frag[NQK > NPV ? NQK : NPV];
+      uint32_t pw[16];
+      const float negm = -m_ref;
+      float la = 0.f, lb = 0.f;
+#pragma unroll
+      for (int j = 0; j < AHEAD; j++) frag[j] = kread(j);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < NQK; j++) {
+        if (j + AHEAD < NQK) frag[j + AHEAD] = kread(j + AHEAD);
+        if (j & 1) n1 = mfma32(frag[j], qf[j >> 1], n1);
+        else n0 = mfma32(frag[j], qf[j >> 1], n0);
+        // exp2 share of this step: 32 / NQK element pairs of S(t)
+#pragma unroll
+        for (int u = 0; u < 16 / NQK; u++) {
+          const int w = j * (16 / NQK) + u;  // pair index 0..15: elements 2w, 2w+1
+          float x0, x1;
+          if (w < 8) { x0 = c0[2 * w]; x1 = c0[2 * w + 1]; } else { x0 = c1[2 * w - 16]; x1 = c1[2 * w - 15]; }
+          x0 = fast_exp2(fmaf(x0, c, negm));
+          x1 = fast_exp2(fmaf(x1, c, negm));
+          la += x0;
+          lb += x1;
+          pw[w] = pack_bf16(x0, x1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      lsum += la + lb;
+      float ma = -INFINITY, mb = -INFINITY;
+      if (!LSE_ONLY) {
+        bf16x8 pb[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++) {
+          u32x4 u = {pw[4 * kb], pw[4 * kb + 1], pw[4 * kb + 2], pw[4 * kb + 3]};
+          pb[kb] = __builtin_bit_cast(bf16x8, u);
+        }
+#pragma unroll
+        for (int j = 0; j < AHEAD; j++) frag[j] = vread(j);
+        __builtin_amdgcn_sched_barrier(0);
+        if (MASKED) mask_tile(n0, n1, nv1);
+#pragma unroll
+        for (int j = 0; j < NPV; j++) {
+          if (j + AHEAD < NPV) frag[j + AHEAD] = vread(j + AHEAD);
+          oacc[j % MTD] = mfma32(frag[j], pb[j / MTD], oacc[j % MTD]);
+          // row-maximum share: spread the 32 elements of S(t+1) over the steps after the first AHEAD
+          constexpr int MSTEPS = NPV - AHEAD;
+          if (j >= AHEAD) {
+            const int e0 = (j - AHEAD) * 16 / MSTEPS, e1 = (j - AHEAD + 1) * 16 / MSTEPS;
+#pragma unroll
+            for (int e = e0; e < e1; e++) {
+              ma = fmaxf(fmaxf(ma, n0[e]), n1[e]);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        if (MASKED) mask_tile(n0, n1, nv1);
+#pragma unroll
+        for (int e = 0; e < 16; e++) ma = fmaxf(fmaxf(ma, n0[e]), n1[e]);
+      }
+      const float mx = xhalf_max(fmaxf(ma, mb));
       __builtin_amdgcn_s_waitcnt(0x0f70);
       __syncthreads();
+      rescale_check(mx);
       nv0 = nv1; nv1 = nv2; nv2 = nv3;
 #pragma unroll
-      for (int s = 0; s < SLOTS; s++) { rows_v[s] = rows_k[s]; rows_k[s] = rows_n[s]; }
+      for (int s = 0; s < NR; s++) { rows_v[s] = rows_k[s]; rows_k[s] = rows_n[s]; }
+    };
+    auto step = [&](int t, auto par, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1) {
+      if (nv1 < 64) body(t, par, std::true_type{}, c0, c1, n0, n1);
+      else body(t, par, std::false_type{}, c0, c1, n0, n1);
+    };
+    // last tile of the list: no successor to prefetch or to multiply
+    auto last = [&](auto par, f32x16& c0, f32x16& c1) {
+      constexpr int PAR = decltype(par)::value;
+      bf16x8 pb[4];
+      exp_tile(c0, c1, pb);
+      if (!LSE_ONLY) pv_tile(pb, smem + (2 + PAR) * TILE);
+      __syncthreads();
     };
 
-    for (int t = 0; t < T; t += 2) {
-      iteration(t, std::integral_constant<int, 0>{}, sa0, sa1, sb0, sb1);
-      if (t + 1 < T) iteration(t + 1, std::integral_constant<int, 1>{}, sb0, sb1, sa0, sa1);
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    int t = 0;
+    for (; t + 2 < T; t += 2) {
+      step(t, P0{}, sa0, sa1, sb0, sb1);
+      step(t + 1, P1{}, sb0, sb1, sa0, sa1);
+    }
+    if (t + 1 < T) {
+      step(t, P0{}, sa0, sa1, sb0, sb1);
+      last(P1{}, sb0, sb1);
+    } else {
+      last(P0{}, sa0, sa1);
     }
   }
 
@@ -311,8 +470,8 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
   AttnParams p = p0;
   constexpr int WGROWS = NWAVES * 32;
   constexpr int SMEM = 4 * 64 * D * 2;
-  if (p.group_rows % WGROWS != 0 && MODE != MODE_DENSE) return LVAR_EINVAL;
-  if (MODE == MODE_DENSE) p.group_rows = WGROWS;
+  if (MODE == MODE_BLOCK && p.list == nullptr) p.group_rows = WGROWS;  // dense: any row grouping
+  if (p.group_rows % WGROWS != 0) return LVAR_EINVAL;
   p.nqt = (p.Lq + WGROWS - 1) / WGROWS;
   p.total_wg = p.B * p.H * p.nqt;
   const int grid = ((p.total_wg + 7) / 8) * 8;
@@ -329,16 +488,14 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
 
 template <int D>
 static int launch_d(const AttnParams& p, int mode, bool accum, bool lse_only, int nwaves, hipStream_t s) {
-  if (mode == MODE_DENSE) {
-    return lse_only ? launch_one<D, 4, MODE_DENSE, false, true>(p, s) : launch_one<D, 4, MODE_DENSE, false, false>(p, s);
-  } else if (mode == MODE_BLOCK) {
-    return launch_one<D, 4, MODE_BLOCK, false, false>(p, s);
-  } else {
+  if (mode == MODE_BLOCK) {
+    return lse_only ? launch_one<D, 4, MODE_BLOCK, false, true>(p, s) : launch_one<D, 4, MODE_BLOCK, false, false>(p, s);
+  } else if (mode == MODE_GATHER) {
     if (nwaves == 6) return launch_one<D, 6, MODE_GATHER, true, false>(p, s);
     if (nwaves == 3) return launch_one<D, 3, MODE_GATHER, true, false>(p, s);
     if (nwaves == 2) return launch_one<D, 2, MODE_GATHER, true, false>(p, s);
-    return LVAR_EUNSUPPORTED;
   }
+  return LVAR_EUNSUPPORTED;
 }
 
 int launch_attn(const AttnParams& p, int head_dim, int mode, bool accum, bool lse_only, int nwaves, hipStream_t s) {

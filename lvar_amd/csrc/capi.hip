@@ -72,7 +72,8 @@ int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_
   p.M = M; p.L = L;
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
   p.c = scale * kLog2e; p.o_scale = 1.f;
-  return launch_attn(p, head_dim, MODE_DENSE, false, lse_only, 4, (hipStream_t)stream);
+  p.list = nullptr; p.cnt = nullptr; p.group_rows = 128; p.sub_shift = 0;
+  return launch_attn(p, head_dim, MODE_BLOCK, false, lse_only, 4, (hipStream_t)stream);
 }
 
 int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* M, const float* L, float* cs,

@@ -7,7 +7,7 @@
 
 namespace lvar {
 
-enum { MODE_DENSE = 0, MODE_BLOCK = 1, MODE_GATHER = 2 };
+enum { MODE_BLOCK = 1, MODE_GATHER = 2 };  // dense attention = MODE_BLOCK with a null list
 
 struct AttnParams {
   const bf16_t *q, *k, *v;
