@@ -121,6 +121,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aux", action="store_true", help="skip the companion dense/colsum/mask-build timings")
     ap.add_argument("--cpu-budget-s", type=float, default=20.0)
+    ap.add_argument("--amp", type=float, default=None, help="override the input amplitude (0 = all-zero inputs, for power experiments)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the hot path on ONE GPU; --gpus N with N > 1 is not supported "
@@ -149,6 +150,8 @@ def main():
         B, H, Lq, Lk, amp = 1, 24, 32768, 32768, 0.5
     else:
         raise SystemExit(f"unknown workload {wl}")
+    if args.amp is not None:
+        amp = args.amp
     q, k, v = make_qkv(B, H, Lq, Lk, d, seed=1234, amp=amp)
     qg, kg, vg = q.to(dev), k.to(dev), v.to(dev)
     scale = 1.0 / math.sqrt(d)

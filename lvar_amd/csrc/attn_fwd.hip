@@ -27,6 +27,9 @@
 
 namespace lvar {
 
+#ifndef LVAR_AHEAD
+#define LVAR_AHEAD 4
+#endif
 static constexpr float RESCALE_TAU = 8.0f;
 static constexpr float NEG_BIG = -1.0e30f;
 
@@ -303,7 +306,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       // compiler from regrouping it.  Phase A: QK MFMA j | K-fragment read j+4 | exp2 of two
       // elements of S(t).  Phase B: PV MFMA j | the two transposing V reads of MFMA j+4 | a slice
       // of the row-maximum reduction of S(t+1).
-      constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = 4;
+      constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = LVAR_AHEAD;
       const char* kbuf = smem + (1 - PAR) * TILE;
       const char* vbuf = smem + (2 + PAR) * TILE;
       auto kread = [&](int j) -> bf16x8 {

@@ -1,0 +1,249 @@
+"""Pins the CPU oracle (oracle/sparse_attn_oracle.py) against things it does not itself define:
+library routines (SDPA, logsumexp, F.interpolate, torch.sort), brute-force pure-Python loops on tiny
+inputs, closed-form special cases and the known answers written in the reference's sources
+(models/sparvar/sparse_attn.py:909,913,934; BASELINE config 1).  The reference ships no golden
+vectors for this path, so these checks are what anchors parity."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+
+
+def rnd(*shape, seed=0, dtype=torch.float64):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=dtype)
+
+
+def test_dense_attn_matches_sdpa_and_logsumexp():
+    q, k, v = rnd(2, 3, 37, 16, seed=1), rnd(2, 3, 53, 16, seed=2), rnd(2, 3, 53, 16, seed=3)
+    for scale in (None, 1.0, 0.3):
+        o, M, L = oracle.dense_attn(q, k, v, scale, dtype=torch.float64)
+        ref = F.scaled_dot_product_attention(q, k, v, scale=scale)
+        assert torch.allclose(o, ref, atol=1e-12)
+        s = oracle.default_scale(16, scale)
+        lse = torch.logsumexp((q @ k.transpose(-1, -2)) * s, dim=-1, keepdim=True)
+        assert torch.allclose(M * math.log(2) + torch.log(L), lse, atol=1e-12)
+        # M is the row maximum of the base-2 logits (attn_dense.py:33-37 masks before the max)
+        assert torch.allclose(M, ((q @ k.transpose(-1, -2)) * s * oracle.LOG2E).max(-1, keepdim=True).values)
+
+
+def test_colsum_bruteforce_tiny():
+    B, H, Lq, Lk, d, G = 1, 1, 40, 13, 4, 32
+    q, k, v = rnd(B, H, Lq, d, seed=4), rnd(B, H, Lk, d, seed=5), rnd(B, H, Lk, d, seed=6)
+    o, cs, _ = oracle.dense_colsum_attn(q, k, v, scale=0.7, q_group_size=G, dtype=torch.float64)
+    exp_cs = [[0.0] * Lk for _ in range((Lq + G - 1) // G)]
+    for i in range(Lq):
+        logits = [0.7 * sum(float(q[0, 0, i, c]) * float(k[0, 0, n, c]) for c in range(d)) for n in range(Lk)]
+        mx = max(logits)
+        e = [math.exp(x - mx) for x in logits]
+        z = sum(e)
+        for n in range(Lk):
+            exp_cs[i // G][n] += e[n] / z
+        row = [sum(e[n] / z * float(v[0, 0, n, c]) for n in range(Lk)) for c in range(d)]
+        assert torch.allclose(o[0, 0, i], torch.tensor(row, dtype=torch.float64), atol=1e-12)
+    assert torch.allclose(cs[0, 0], torch.tensor(exp_cs, dtype=torch.float64), atol=1e-12)
+
+
+def test_colsum_invariants_and_special_cases():
+    B, H, Lq, Lk, d = 2, 2, 300, 77, 8
+    q, k, v = rnd(B, H, Lq, d, seed=7), rnd(B, H, Lk, d, seed=8), rnd(B, H, Lk, d, seed=9)
+    _, cs, (M, L) = oracle.dense_colsum_attn(q, k, v, dtype=torch.float64)
+    assert cs.shape == (B, H, 2, Lk) and bool((cs >= 0).all())
+    # each softmax row sums to one: the last group has 300 - 192 = 108 rows (rows >= Lq add zero)
+    assert torch.allclose(cs.sum(-1), torch.tensor([192.0, 108.0], dtype=torch.float64).expand(B, H, 2))
+    _, cs_all, _ = oracle.dense_colsum_attn(q, k, v, q_group_size=Lq, dtype=torch.float64)
+    assert torch.allclose(cs.sum(2, keepdim=True), cs_all, atol=1e-12)
+    # second pass given (M, L) reproduces the fused result
+    assert torch.allclose(oracle.colsum_from_lse(q, k, M, L, dtype=torch.float64), cs, atol=1e-12)
+    # q = 0 => uniform rows => cs = rows / Lk
+    _, cs0, _ = oracle.dense_colsum_attn(torch.zeros_like(q), k, v, dtype=torch.float64)
+    assert torch.allclose(cs0[:, :, 0], torch.full((B, H, Lk), 192.0 / Lk, dtype=torch.float64))
+    # the reference's own PyTorch statement of the op (sparse_attn_ops.py:179-200), retyped from its
+    # formula with library calls only
+    attn = torch.softmax(q @ k.transpose(-2, -1) / math.sqrt(d), dim=-1)
+    pad = F.pad(attn, (0, 0, 0, 2 * 192 - Lq)).view(B, H, 2, 192, Lk).sum(3)
+    assert torch.allclose(cs, pad, atol=1e-12)
+
+
+def test_key_block_sums_ragged():
+    cs = torch.arange(680, dtype=torch.float64).view(1, 1, 1, 680)
+    bs = oracle.key_block_sums(cs, 64)
+    assert bs.shape[-1] == 11
+    assert bs[0, 0, 0, 0] == sum(range(64)) and bs[0, 0, 0, 10] == sum(range(640, 680))
+
+
+def test_indices_count_known_answers():
+    # decision scale of Infinity-2B: Lk = 4121, top_keys = 0.2 (sparse-attn-config.yml:20)
+    assert oracle.indices_count(0.2, 4121, 64) == 832
+    assert oracle.indices_count(0.2, 4121, 112) == 784
+    # BASELINE config 1: Lk = 680, keep 50 % => 320 tokens = 5 blocks of 64
+    assert oracle.indices_count(0.5, 680, 64) == 320
+    # half-to-even: 0.25*640/64 = 2.5 -> 2
+    assert oracle.indices_count(0.25, 640, 64) == 128
+    assert oracle.infinity_cum() == [0, 1, 5, 21, 57, 121, 265, 521, 921, 1497, 2521, 4121, 6425, 10521]
+
+
+def test_topk_index_list_is_the_sorted_prefix():
+    bs = rnd(1, 2, 3, 200, seed=10).abs()
+    inds, counts = oracle.topk_index_list(bs, 0.3, multiple_of=16)
+    cnt = 16 * round(0.3 * 200 / 16)
+    assert inds.shape == (1, 2, 3, 200) and inds.dtype == torch.int32 and int(counts[0, 0, 0]) == cnt
+    order = torch.sort(bs, dim=-1, descending=True, stable=True).indices[..., :cnt]
+    assert torch.equal(inds[..., :cnt].long(), order)  # values are distinct, so the order is fixed
+
+
+def _gather_attention_bruteforce(q, k, v, idx, scale):
+    out = []
+    for i in range(q.shape[0]):
+        logits = [scale * float(q[i] @ k[j]) for j in idx]
+        mx = max(logits)
+        e = [math.exp(x - mx) for x in logits]
+        z = sum(e)
+        out.append(sum((e[t] / z) * v[j] for t, j in enumerate(idx)))
+    return torch.stack(out)
+
+
+def test_csp_attn_multiset_semantics():
+    B, H, Lq, Lk, d, bm = 1, 2, 50, 30, 4, 32
+    q, k, v = rnd(B, H, Lq, d, seed=11), rnd(B, H, Lk, d, seed=12), rnd(B, H, Lk, d, seed=13)
+    G = 2
+    inds = torch.zeros(B, H, G, Lk, dtype=torch.int32)
+    counts = torch.zeros(B, H, G, dtype=torch.int32)
+    lists = {(0, 0): [3, 3, 7, 29, 0], (0, 1): [5], (1, 0): list(range(30)), (1, 1): []}
+    for (h, g), l in lists.items():
+        inds[0, h, g, :len(l)] = torch.tensor(l, dtype=torch.int32)
+        counts[0, h, g] = len(l)
+    delta, M, L = oracle.csp_attn_delta(q, k, v, inds, counts, scale=0.5, bm=bm, dtype=torch.float64)
+    for (h, g), l in lists.items():
+        lo, hi = g * bm, min((g + 1) * bm, Lq)
+        if not l:
+            assert bool((delta[0, h, lo:hi] == 0).all()) and bool(torch.isinf(M[0, h, lo:hi]).all()) and bool((L[0, h, lo:hi] == 1).all())
+            continue
+        ref = _gather_attention_bruteforce(q[0, h, lo:hi], k[0, h], v[0, h], l, 0.5)
+        assert torch.allclose(delta[0, h, lo:hi], ref, atol=1e-12)
+    # full list == dense attention (attn_csp.py:313-338); o_scale epilogue (attn_csp.py:209-211)
+    dense, _, _ = oracle.dense_attn(q[:, 1:2], k[:, 1:2], v[:, 1:2], 0.5, dtype=torch.float64)
+    assert torch.allclose(delta[0, 1, :bm], dense[0, 0, :bm], atol=1e-12)
+    o0 = rnd(B, H, Lq, d, seed=14)
+    assert torch.allclose(oracle.csp_attn(q, k, v, 0.5, inds, counts, o0, -1, bm=bm, dtype=torch.float64), o0 - delta)
+
+
+def test_csp_unique_list_equals_masked_softmax():
+    """The reference's own oracle form (attn_csp.py:437-471): dense softmax, unselected logits -> -1e9."""
+    B, H, Lq, Lk, d = 1, 1, 192, 64, 8
+    q, k, v = rnd(B, H, Lq, d, seed=15), rnd(B, H, Lk, d, seed=16), rnd(B, H, Lk, d, seed=17)
+    sel = torch.randperm(Lk, generator=torch.Generator().manual_seed(1))[:20]
+    inds = torch.zeros(B, H, 1, Lk, dtype=torch.int32)
+    inds[0, 0, 0, :20] = sel.to(torch.int32)
+    counts = torch.full((B, H, 1), 20, dtype=torch.int32)
+    delta, _, _ = oracle.csp_attn_delta(q, k, v, inds, counts, dtype=torch.float64)
+    logits = (q @ k.transpose(-1, -2)) / math.sqrt(d)
+    mask = torch.zeros(Lk, dtype=torch.bool)
+    mask[sel] = True
+    ref = torch.softmax(logits.masked_fill(~mask, -1e9), -1) @ v
+    assert torch.allclose(delta, ref, atol=1e-12)
+
+
+def test_block_sparse_equals_masked_dense():
+    B, H, Lq, Lk, d, bq, bk = 1, 2, 200, 150, 8, 128, 64
+    q, k, v = rnd(B, H, Lq, d, seed=18), rnd(B, H, Lk, d, seed=19), rnd(B, H, Lk, d, seed=20)
+    mask = torch.tensor([[[1, 0, 1], [0, 1, 1]], [[0, 0, 1], [1, 1, 1]]], dtype=torch.bool).view(1, 2, 2, 3)
+    num, idx = oracle.block_mask_to_lists(mask)
+    assert num.tolist() == [[[2, 2], [1, 3]]] and idx[0, 0, 0, :2].tolist() == [0, 2]
+    assert torch.equal(oracle.lists_to_block_mask(num, idx, 3), mask)
+    o, M, L = oracle.block_sparse_attn(q, k, v, num, idx, bq, bk, dtype=torch.float64)
+    fine = mask.repeat_interleave(bq, 2).repeat_interleave(bk, 3)[:, :, :Lq, :Lk]
+    logits = (q @ k.transpose(-1, -2)) / math.sqrt(d)
+    ref = torch.softmax(logits.masked_fill(~fine, -float("inf")), -1) @ v
+    assert torch.allclose(o, ref, atol=1e-12)
+    lse = torch.logsumexp(logits.masked_fill(~fine, -float("inf")), -1, keepdim=True)
+    assert torch.allclose(M * math.log(2) + torch.log(L), lse, atol=1e-12)
+    assert oracle.attn_flops_blocks(num, idx, Lq, Lk, d, bq, bk) == 4 * d * int(fine.sum())
+
+
+def test_map_inds_counts_across_scales_bruteforce():
+    # Gs = 9 (decision scale, 1600 rows), target scales 11 (2304 rows, G=12) and 12 (4096 rows, G=22)
+    g = torch.Generator().manual_seed(3)
+    inds_S = torch.randint(0, 4121, (2, 2, 9, 4121), generator=g, dtype=torch.int32)
+    counts_S = torch.full((2, 2, 9), 832, dtype=torch.int32)
+    for q_len, k_len in ((2304, 6425), (4096, 10521)):
+        out, counts = oracle.map_inds_counts_across_scales(inds_S, counts_S, q_len, k_len)
+        Gk = (q_len + 191) // 192
+        assert out.shape == (2, 2, Gk, 832) and bool((counts == 832).all())
+        for gk in range(Gk):
+            gs = min(max(round((gk + 0.5) / Gk * 9 - 0.5), 0), 8)  # python round = half-to-even
+            assert torch.equal(out[:, :, gk], inds_S[:, :, gs, :832])
+    # narrower source than the padded count: cyclic repeat_interleave, then clamp to the key range
+    small = torch.tensor([5, 9, 100], dtype=torch.int32).view(1, 1, 1, 3)
+    out, counts = oracle.map_inds_counts_across_scales(small, torch.tensor([[[3]]]), 192, 50, indices_pad_to=4)
+    assert out.tolist() == [[[[5, 5, 9, 9]]]] and int(counts[0, 0, 0]) == 4
+    out, _ = oracle.map_inds_counts_across_scales(small, torch.tensor([[[3]]]), 192, 50)
+    assert out.tolist() == [[[[5, 9, 49]]]]
+
+
+def test_local_window_runs_known_answers():
+    """Source comment models/sparvar/sparse_attn.py:934: windows (5, 7), counts_multiple_of 112
+    -> scale 11: [12, 448], scale 12: [22, 672]."""
+    for si, win, shape in ((11, 5, (12, 448)), (12, 7, (22, 672))):
+        ia, kv = oracle.crossscale_self_indices(si, win)
+        S = oracle.INFINITY_SCALES[si]
+        assert ia.shape[0] == S * S and kv == oracle.infinity_cum()[si + 1]
+        runs, L = oracle.aggregate_group_indices(ia, S * S, kv, 192, 112)
+        assert tuple(runs.shape) == shape and L == shape[1]
+        assert bool((runs[:, 1:] - runs[:, :-1] == 1).all())                  # contiguous runs
+        assert int(runs.min()) >= oracle.infinity_cum()[si] and int(runs.max()) == kv - 1
+    # interior query of an 8x8 grid, 3x3 window: the 9 neighbours, row-major
+    w = oracle.local_window_indices(8, 8, 100, 3)
+    assert w[9].tolist() == [100, 101, 102, 108, 109, 110, 116, 117, 118]
+    assert w[0].tolist() == [100, 100, 101, 100, 100, 101, 108, 108, 109]     # clamp padding at the corner
+
+
+def test_upsample_ocache_matches_interpolate():
+    x = rnd(2, 3, 40 * 40, 8, seed=21)
+    for tgt in (48, 64):
+        got = oracle.upsample_ocache(x, 1600, tgt * tgt)
+        ref = F.interpolate(x.view(2, 3, 40, 40, 8).permute(0, 1, 4, 2, 3).reshape(6, 8, 40, 40), size=(tgt, tgt),
+                            mode="bilinear", align_corners=False)
+        ref = ref.view(2, 3, 8, tgt, tgt).permute(0, 1, 3, 4, 2).reshape(2, 3, tgt * tgt, 8)
+        assert torch.allclose(got, ref, atol=1e-10)
+
+
+def test_flex_block_mask_properties():
+    # scale index 8 (24x24 queries, 1497 keys) keeps the pure-Python brute force fast
+    ks = [-1, -1, -1, -1, 1, 1, 3, 5, 7]
+    m = oracle.flex_block_mask(8, ks, 3, 128)
+    cum = oracle.infinity_cum()
+    assert m.shape == ((576 + 127) // 128, (cum[9] + 127) // 128)
+    assert bool(m[:, 0].all())                       # sink: keys < cum[3] = 21 are in block 0
+    # hand check of one fine-grained entry: query (12, 12) of the 24x24 grid looks at the 16x16 scale
+    # (index 6, kernel 3) around round(12/24*16) = 8: keys (7..9, 7..9); key (8, 8) = cum[6] + 8*16 + 8
+    kv = cum[6] + 8 * 16 + 8
+    assert bool(m[(12 * 24 + 12) // 128, kv // 128])
+    # negative kernel size: a scale beyond the sink is never attended.  Scale 3 (keys 21..56) has
+    # kernel -1; with 32-wide key blocks, block 1 (keys 32..63) holds scale 3 and the head of scale 4
+    m32 = oracle.flex_block_mask(8, [-1] * 9, 3, 128, block_k=32)
+    assert bool(m32[:, 0].all()) and not bool(m32[:, 1:].any())
+    # mixed block shape (128 x 64) is the same predicate reduced over other tiles
+    m2 = oracle.flex_block_mask(8, ks, 3, 128, block_k=64)
+    pad = F.pad(m2, (0, m2.shape[1] % 2))
+    assert torch.equal(pad.view(pad.shape[0], -1, 2).any(-1), m)
+
+
+def test_config2_block_mask_density():
+    scores = rnd(1, 2, 32, 165, seed=22).abs()
+    mask = oracle.config2_block_mask(scores)
+    assert mask.shape == (1, 2, 32, 165)
+    target = round(0.25 * 165)
+    assert bool((mask.sum(-1) == target).all())
+    assert bool(mask[..., :9].all())                 # keys < 521 -> blocks 0..8 always kept
+    # the score-independent part, and the score-selected remainder = best remaining blocks
+    base = oracle.config2_block_mask(scores, density=0.0)
+    assert bool((base[0, 0] == base[0, 1]).all()) and bool((mask | ~base).all())
+    for h in range(2):
+        for i in range(32):
+            extra = (mask[0, h, i] & ~base[0, h, i]).nonzero().flatten()
+            rest = scores[0, h, i].masked_fill(base[0, h, i], -1.0)
+            best = torch.sort(rest, descending=True).indices[:extra.numel()]
+            assert sorted(extra.tolist()) == sorted(best.tolist())
