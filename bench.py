@@ -205,10 +205,10 @@ def main():
             cpu = {"value": round(dense_flops / (B * H) * done / t / 1e12, 5), "unit": "TFLOP/s", "cores": os.cpu_count(),
                    "kind": "port", "sample": f"{done} of {B * H} (batch,head) slices, {t:.1f} s"}
     elif wl in ("colsum", "colsum_scale48"):
-        M, L = ops._lse_only(qg, kg, scale)
-        flops = 2.0 * B * H * Lq * Lk * d      # column sweep with (M, L) supplied
-        fn = lambda: ops._colsum_given_lse(qg, kg, M, L, scale, 192)
-        kernel = "colsum_kernel<128,2>"
+        lse2 = ops._lse_only(qg, kg, scale)
+        flops = 2.0 * B * H * Lq * Lk * d      # column sweep with the row statistics supplied
+        fn = lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 192)
+        kernel = "colsum_kernel<128>"
         config["form"] = "one-pass given (M,L): 2*B*H*Lq*Lk*d flops"
         if not args.no_cpu_baseline:
             done, t = cpu_baseline_dense(q, k, v, args.cpu_budget_s, colsum=True)
@@ -233,13 +233,13 @@ def main():
     if wl == "block_sparse_25" and not args.no_aux:
         # companion numbers named by the metric: colsum (+ mask build) versus the dense attention it replaces
         dense_ms, _ = time_launches(lambda: ops.dense_attn(qg, kg, vg, scale), 10, 3)
-        M, L = ops._lse_only(qg, kg, scale)
-        cs_ms, _ = time_launches(lambda: ops._colsum_given_lse(qg, kg, M, L, scale, 128), 10, 3)
+        lse2 = ops._lse_only(qg, kg, scale)
+        cs_ms, _ = time_launches(lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 128), 10, 3)
         lse_ms, _ = time_launches(lambda: ops._lse_only(qg, kg, scale), 10, 3)
 
         def build():
-            cs = ops._colsum_given_lse(qg, kg, M, L, scale, 128)
-            return mb.block_mask_to_lists(mb.sink_window_topk_block_mask(mb.key_block_sums(cs, 64), 128, 64, 0.25))
+            _, bs = ops._colsum_given_lse(qg, kg, lse2, scale, 128, want_block_sums=True)
+            return mb.block_mask_to_lists(mb.sink_window_topk_block_mask(bs, 128, 64, 0.25))
         build_ms, _ = time_launches(build, 5, 2)
         aux = {"dense_attn_ms": round(dense_ms, 4), "dense_attn_tflops": round(dense_flops / dense_ms / 1e9, 1),
                "colsum_given_lse_us": round(cs_ms * 1e3, 1), "lse_pass_us": round(lse_ms * 1e3, 1),

@@ -43,23 +43,28 @@ const char* lvar_status_string(int status);
  * Replaces torch.ops.chipmunk.dense_attn (kernels/chipmunk/csrc/chipmunk.cu:57,
  * kernels/chipmunk/csrc/attn/dense_attn.cu:248-372) and sattn_triton.dense_attn
  * (kernels/sparse_attn/triton/attn_dense.py:186-231).
- * o may be NULL (statistics only); M and L may be NULL.  head_dim in {64, 128}.
+ * LSE2, if not NULL, receives the base-2 log-sum-exp M + log2(L) (fp32 [B,H,Lq]), the form the
+ * colsum entry point consumes.  o may be NULL (statistics only); M, L and LSE2 may each be NULL.
+ * head_dim in {64, 128}.
  */
 int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o,
-                        float* M, float* L,
+                        float* M, float* L, float* LSE2,
                         int B, int H, int Lq, int Lk, int head_dim,
                         float scale, void* stream);
 
 /*
- * Colsum given (M, L): cs[b,h,g,n] = sum_{i in group g} exp2(q_i.k_n*scale*log2e - M_i)/L_i,
- * groups of q_group_size consecutive query rows (multiple of 32), rows >= Lq add zero.
- * cs is fp32 contiguous [B,H,ceil(Lq/q_group_size),Lk]; every element is written exactly
- * once (no atomics, no pre-zeroing needed, deterministic).
+ * Colsum given the row statistics: cs[b,h,g,n] = sum_{i in group g} exp2(q_i.k_n*scale*log2e - lse2_i),
+ * lse2 = M + log2(L) (fp32 contiguous [B,H,Lq], as written by lvar_dense_attn_fwd), groups of
+ * q_group_size consecutive query rows (a multiple of 32), rows >= Lq add zero.
+ * cs is fp32 contiguous [B,H,G,Lk], G = ceil(Lq/q_group_size); every element is written exactly once
+ * (no atomics, no pre-zeroing, deterministic).  block_sums, if not NULL, receives the sums of cs over
+ * blocks of 64 consecutive keys, fp32 contiguous [B,H,G,ceil(Lk/64)] (ragged last block).
  * Replaces pass 2 of _full_attn_fwd (kernels/sparse_attn/triton/attn_dense_colsum.py:216-231)
  * and torch.ops.chipmunk.dense_colsum_attn (kernels/chipmunk/csrc/chipmunk.cu:58,
- * kernels/chipmunk/csrc/attn/dense_colsum_attn.cu:355-522).
+ * kernels/chipmunk/csrc/attn/dense_colsum_attn.cu:355-522), which takes the same precomputed
+ * per-row constant as its fourth argument.
  */
-int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* M, const float* L, float* cs,
+int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* cs, float* block_sums,
                     int B, int H, int Lq, int Lk, int head_dim, int q_group_size,
                     float scale, void* stream);
 

@@ -425,6 +425,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     const int64_t off = ((int64_t)b * p.H + h) * p.Lq + qrow_w;
     if (p.M) p.M[off] = empty ? -INFINITY : m_true;
     if (p.L) p.L[off] = empty ? 1.0f : ltot * fast_exp2(m_ref - m_true);
+    if (p.LSE2) p.LSE2[off] = empty ? -INFINITY : m_ref + __builtin_amdgcn_logf(ltot);
   }
   if (LSE_ONLY) return;
 

@@ -60,30 +60,31 @@ const char* lvar_status_string(int status) {
 }
 
 int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
-                        int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
+                        float* LSE2, int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k)) return LVAR_EINVAL;
   const bool lse_only = (o.ptr == nullptr);
   if (!kv_span_ok(k, Lk, head_dim) || (!lse_only && !kv_span_ok(v, Lk, head_dim))) return LVAR_EINVAL;
   if (!lse_only && (!view_ok(v) || !view_ok(o))) return LVAR_EINVAL;
-  if (lse_only && !(M && L)) return LVAR_EINVAL;
+  if (lse_only && !((M && L) || LSE2)) return LVAR_EINVAL;
   AttnParams p{};
   fill_qkv(p, q, k, lse_only ? k : v);
   p.o = (bf16_t*)o.ptr; p.o_sb = o.stride_b; p.o_sh = o.stride_h; p.o_sr = o.stride_row;
-  p.M = M; p.L = L;
+  p.M = M; p.L = L; p.LSE2 = LSE2;
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
   p.c = scale * kLog2e; p.o_scale = 1.f;
   p.list = nullptr; p.cnt = nullptr; p.group_rows = 128; p.sub_shift = 0;
   return launch_attn(p, head_dim, MODE_BLOCK, false, lse_only, 4, (hipStream_t)stream);
 }
 
-int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* M, const float* L, float* cs,
+int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* cs, float* block_sums,
                     int B, int H, int Lq, int Lk, int head_dim, int q_group_size, float scale, void* stream) {
-  if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !M || !L || !cs) return LVAR_EINVAL;
+  if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !lse2 || !cs) return LVAR_EINVAL;
   if (q_group_size <= 0 || q_group_size % 32 != 0) return LVAR_EINVAL;
+  if (!kv_span_ok(q, Lq, head_dim)) return LVAR_EINVAL;
   ColsumParams p{};
   p.q = (const bf16_t*)q.ptr; p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sr = q.stride_row;
   p.k = (const bf16_t*)k.ptr; p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sr = k.stride_row;
-  p.M = M; p.L = L; p.cs = cs;
+  p.lse2 = lse2; p.cs = cs; p.bs = block_sums;
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
   p.group_rows = q_group_size;
   p.G = (Lq + q_group_size - 1) / q_group_size;

@@ -1,148 +1,241 @@
 // Colsum kernel for gfx950: cs[b,h,g,n] = sum over the query rows i of group g of
-// exp2(q_i.k_n*scale*log2e - lse2_i), lse2 = M + log2(L).
+// exp2(q_i.k_n*scale*log2e - lse2_i), with lse2 = M + log2(L) the base-2 log-sum-exp of row i.
 //
-// Key-stationary decomposition: a wave keeps NTK*32 keys (the B operand, K^T) in registers for
-// the whole sweep over Lq, the workgroup streams 64-row Q stages (+ their lse2) through LDS as
-// the A operand.  In the 32x32 accumulator a lane owns ONE key column and 16 query rows, so the
-// reduction over queries is an in-register add, one exchange with lane^32 at each group
-// boundary, and a single plain store per (group, key): no atomics, no partial buffers, and a
-// summation order that depends only on the shapes.
+// Key-stationary decomposition: a wave keeps one 64-key block (the B operand, K^T) in registers
+// for the whole sweep over Lq; the workgroup (4 waves = 256 keys) streams 64-row Q stages and their
+// lse2 through a 4-deep LDS ring filled by global->LDS DMA three stages ahead.  In the 32x32
+// accumulator a lane owns ONE key column and 16 query rows, so the reduction over queries is an
+// in-register add, one exchange with lane^32 at each group boundary and a single plain store per
+// (group, key): no atomics, no partial buffers, and a summation order fixed by the shapes alone.
+// The per-64-key block sums fall out of the same registers (one wave = one key block).
+//
+// Inner loop, software-pipelined by hand: while the matrix cores compute S(u) = Q_tile(u) K^T for
+// 32-row tile u (16 MFMA for d = 128), the vector ALU turns S(u-1) into probabilities and adds them
+// to the column accumulators.
+#include <type_traits>
 #include "common.h"
 #include "launch.h"
 
 namespace lvar {
 
-template <int D, int NTK>
+template <int D>
 __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
-  constexpr int KS = D / 16, CPR = D / 8;
-  constexpr int QSTR = D * 2 + 16;
-  constexpr int QROWS = 64;
-  constexpr int CPT = (QROWS * CPR) / 256;
-  constexpr int STAGE = QROWS * QSTR + QROWS * 4;
-  __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int KS = D / 16;
+  constexpr int ROWB = D * 2, CPR = ROWB / 16;
+  constexpr int RPI = 1024 / ROWB, NI = 64 / RPI, SLOTS = NI / 4;
+  constexpr int QTILE = 64 * ROWB;         // one 64-row Q stage
+  constexpr int NSTAGE = 4, NLSE = 8;      // ring depths
+  constexpr int LSE_OFF = NSTAGE * QTILE;  // lse2 ring: NLSE x 64 floats
+  extern __shared__ __attribute__((aligned(1024))) char smem[];  // NSTAGE * QTILE + NLSE * 256 bytes
 
   const int per_xcd = gridDim.x >> 3;
   const int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (w >= p.total_wg) return;
   const int bh = w / p.nkt, kt = w - bh * p.nkt;
   const int b = bh / p.H, h = bh - b * p.H;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, r = lane & 31;
-  const int n0 = (kt * 4 + wave) * (NTK * 32);
+  const int kblk = kt * 4 + wave;  // 64-key block owned by this wave
+  const int n0 = kblk * 64;
+  const float c = p.c;
 
-  // stationary K^T fragments
+  // stationary K^T fragments: lane holds key column n0 + nt*32 + r, d = ks*16 + 8*hh .. +7
   const bf16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
-  bf16x8 kf[NTK][KS];
+  bf16x8 kf[2][KS];
 #pragma unroll
-  for (int nt = 0; nt < NTK; nt++) {
+  for (int nt = 0; nt < 2; nt++) {
     const int krow = min(n0 + nt * 32 + r, p.Lk - 1);
     const bf16_t* kp = kbase + (int64_t)krow * p.k_sr + hh * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) kf[nt][ks] = *(const bf16x8*)(kp + ks * 16);
   }
 
-  const bf16_t* qbase = p.q + b * p.q_sb + h * p.q_sh;
-  const float* Mp = p.M + ((int64_t)b * p.H + h) * p.Lq;
-  const float* Lp = p.L + ((int64_t)b * p.H + h) * p.Lq;
+  auto make_rsrc = [](const void* base) -> i32x4 {
+    const uint64_t a = (uint64_t)base;
+    i32x4 rs = {__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
+                __builtin_amdgcn_readfirstlane((int)(uint32_t)((a >> 32) & 0xffffu)), 0x7fffffff, 0x00020000};
+    return rs;
+  };
+  const i32x4 qrsrc = make_rsrc(p.q + b * p.q_sb + h * p.q_sh);
+  const i32x4 lrsrc = make_rsrc(p.lse2 + ((int64_t)b * p.H + h) * p.Lq);
+  const int q_srb = (int)p.q_sr * 2;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(LVAR_LDS char*)smem;
+  const int lrow = lane / CPR, lcs = lane % CPR;
+
+  // global->LDS fill of stage s (Q rows s*64 .. +63, clamped to Lq-1, chunk-swizzled; lse2 by wave 0)
+  auto issue_stage = [&](int s) {
+    const uint32_t dst = lds0 + (s & (NSTAGE - 1)) * QTILE;
+#pragma unroll
+    for (int sl = 0; sl < SLOTS; sl++) {
+      const int i = wave + sl * 4;
+      const int trow = i * RPI + lrow;
+      const int grow = min(s * 64 + trow, p.Lq - 1);
+      const int voff = grow * q_srb + ((lcs ^ ((trow / (256 / ROWB)) & (CPR - 1))) << 4);
+      const uint32_t m0v = dst + i * 1024;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(m0v), "v"(voff), "s"(qrsrc) : "memory");
+    }
+    if (wave == 0) {
+      const int voff = min(s * 64 + lane, p.Lq - 1) * 4;
+      const uint32_t m0v = lds0 + LSE_OFF + (s & (NLSE - 1)) * 256;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(m0v), "v"(voff), "s"(lrsrc) : "memory");
+    }
+  };
+  // wait until at most `younger` later stages of this wave's fills are still in flight
+  auto wait_fills = [&](int younger) {
+    if (younger >= 2) {
+      if (wave == 0) __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * (SLOTS + 1))); else __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * SLOTS));
+    } else if (younger == 1) {
+      if (wave == 0) __builtin_amdgcn_s_waitcnt(0x0f70 | (SLOTS + 1)); else __builtin_amdgcn_s_waitcnt(0x0f70 | SLOTS);
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+    }
+  };
+
   float* csp = p.cs + ((int64_t)b * p.H + h) * p.G * (int64_t)p.Lk;
-
-  int crow[CPT], ccol[CPT];
+  float* bsp = p.bs ? p.bs + ((int64_t)b * p.H + h) * p.G * (int64_t)p.nkb : nullptr;
+  // store the finished column sums of group g and reset the accumulators
+  auto flush = [&](int g, float (&acc)[2]) {
+    float blk = 0.f;
 #pragma unroll
-  for (int i = 0; i < CPT; i++) {
-    int c = tid + i * 256;
-    crow[i] = c / CPR;
-    ccol[i] = c - crow[i] * CPR;
-  }
-  u32x4 qreg[CPT];
-  float lsereg = 0.f;
-  auto load_stage = [&](int s) {
-    const int base = s * QROWS;
-#pragma unroll
-    for (int i = 0; i < CPT; i++) {
-      const int row = min(base + crow[i], p.Lq - 1);
-      qreg[i] = *(const u32x4*)(qbase + (int64_t)row * p.q_sr + ccol[i] * 8);
+    for (int nt = 0; nt < 2; nt++) {
+      const float tot = xhalf_sum(acc[nt]);
+      const int key = n0 + nt * 32 + r;
+      const bool ok = key < p.Lk;
+      if (hh == 0 && ok) csp[(int64_t)g * p.Lk + key] = tot;
+      blk += ok ? tot : 0.f;
+      acc[nt] = 0.f;
     }
-    if (tid < QROWS) {
-      const int row = base + tid;
-      lsereg = (row < p.Lq) ? Mp[row] + __builtin_amdgcn_logf(Lp[row]) : INFINITY;
+    if (bsp) {
+#pragma unroll
+      for (int m = 16; m >= 1; m >>= 1) blk += __shfl_xor(blk, m);
+      if (lane == 0 && n0 < p.Lk) bsp[(int64_t)g * p.nkb + kblk] = blk;
     }
   };
-  auto store_stage = [&](int st) {
-    char* qs = smem + st * STAGE;
+
+  const int S = (p.Lq + 63) >> 6;          // stages
+  const int U = (p.Lq + 31) >> 5;          // 32-row tiles
+  const int kbase_l = r * ROWB + ((hh ^ ((r / (256 / ROWB)) & (CPR - 1))) << 4);
+  float acc[2] = {0.f, 0.f};
+
+  // probabilities of tile u from its logits: p = exp2(s*c - lse2[row]); rows >= Lq add nothing
+  auto exp_acc = [&](int u, const f32x16& s0, const f32x16& s1) {
+    const char* ll = smem + LSE_OFF + ((u >> 1) & (NLSE - 1)) * 256 + ((u & 1) * 32 + 4 * hh) * 4;
+    f32x4 lse[4];
 #pragma unroll
-    for (int i = 0; i < CPT; i++) *(u32x4*)(qs + crow[i] * QSTR + ccol[i] * 16) = qreg[i];
-    if (tid < QROWS) *(float*)(qs + QROWS * QSTR + tid * 4) = lsereg;
+    for (int j = 0; j < 4; j++) lse[j] = *(const f32x4*)(ll + j * 32);
+    const bool ragged = (u * 32 + 32 > p.Lq);
+    const int lim = p.Lq - u * 32 - 4 * hh;
+    float pa = 0.f, pb = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      float x0 = fast_exp2(fmaf(s0[i], c, -lse[i >> 2][i & 3]));
+      float x1 = fast_exp2(fmaf(s1[i], c, -lse[i >> 2][i & 3]));
+      if (ragged) {
+        const bool ok = (8 * (i >> 2) + (i & 3)) < lim;
+        x0 = ok ? x0 : 0.f;
+        x1 = ok ? x1 : 0.f;
+      }
+      pa += x0;
+      pb += x1;
+    }
+    acc[0] += pa;
+    acc[1] += pb;
+    const int qend = u * 32 + 32;
+    if (qend % p.group_rows == 0 || qend >= p.Lq) flush((u * 32) / p.group_rows, acc);
   };
 
-  const int S = (p.Lq + QROWS - 1) / QROWS;
-  const float c = p.c;
-  float acc[NTK];
-#pragma unroll
-  for (int nt = 0; nt < NTK; nt++) acc[nt] = 0.f;
-
-  load_stage(0);
-  store_stage(0);
+  // prologue: up to three stages in flight
+  issue_stage(0);
+  if (S > 1) issue_stage(1);
+  if (S > 2) issue_stage(2);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
   __syncthreads();
 
-  for (int s = 0; s < S; s++) {
-    const int st = s & 1;
-    if (s + 1 < S) load_stage(s + 1);
-    const char* qs = smem + st * STAGE;
+  // One pipelined step: S(u) -> (n0, n1) on the matrix cores, probabilities of tile u-1 from (c0, c1)
+  // on the vector ALU, interleaved by hand (sched_barrier(0) pins each group).
+  auto step = [&](int u, f32x16& n0a, f32x16& n1a, const f32x16& c0, const f32x16& c1, bool have_prev) {
+    const char* qb = smem + ((u >> 1) & (NSTAGE - 1)) * QTILE + (u & 1) * 32 * ROWB;
+    constexpr int AHEAD = 3;
+    bf16x8 frag[KS];
 #pragma unroll
-    for (int qt = 0; qt < 2; qt++) {
-      const int qrow0 = s * QROWS + qt * 32;
-      if (qrow0 < p.Lq) {
-        bf16x8 a[KS];
-        const char* ql = qs + (qt * 32 + r) * QSTR + hh * 16;
+    for (int i = 0; i < 16; i++) { n0a[i] = 0.f; n1a[i] = 0.f; }
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) a[ks] = *(const bf16x8*)(ql + ks * 32);
-        f32x4 lse[4];
-        const char* ll = qs + QROWS * QSTR + (qt * 32 + 4 * hh) * 4;
+    for (int j = 0; j < AHEAD && j < KS; j++) frag[j] = *(const bf16x8*)(qb + (kbase_l ^ (j << 5)));
+    if (have_prev) {
+      const int up = u - 1;
+      const char* ll = smem + LSE_OFF + ((up >> 1) & (NLSE - 1)) * 256 + ((up & 1) * 32 + 4 * hh) * 4;
+      f32x4 lse[4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) lse[j] = *(const f32x4*)(ll + j * 32);
+      for (int j = 0; j < 4; j++) lse[j] = *(const f32x4*)(ll + j * 32);
+      float pa = 0.f, pb = 0.f;
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int nt = 0; nt < NTK; nt++) {
-          f32x16 sacc;
+      for (int ks = 0; ks < KS; ks++) {
+        if (ks + AHEAD < KS) frag[ks + AHEAD] = *(const bf16x8*)(qb + (kbase_l ^ ((ks + AHEAD) << 5)));
+        n0a = mfma32(frag[ks], kf[0][ks], n0a);
+        n1a = mfma32(frag[ks], kf[1][ks], n1a);
+        // share of the exp work: 16 / KS accumulator indices of both key tiles
 #pragma unroll
-          for (int i = 0; i < 16; i++) sacc[i] = 0.f;
-#pragma unroll
-          for (int ks = 0; ks < KS; ks++) sacc = mfma32(a[ks], kf[nt][ks], sacc);
-          float part = 0.f;
-#pragma unroll
-          for (int i = 0; i < 16; i++) part += fast_exp2(fmaf(sacc[i], c, -lse[i >> 2][i & 3]));
-          acc[nt] += part;
+        for (int e = 0; e < 16 / KS; e++) {
+          const int i = ks * (16 / KS) + e;
+          pa += fast_exp2(fmaf(c0[i], c, -lse[i >> 2][i & 3]));
+          pb += fast_exp2(fmaf(c1[i], c, -lse[i >> 2][i & 3]));
         }
-        const int qend = qrow0 + 32;
-        if (qend % p.group_rows == 0 || qend >= p.Lq) {
-          const int g = qrow0 / p.group_rows;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      acc[0] += pa;
+      acc[1] += pb;
+      const int qend = up * 32 + 32;
+      if (qend % p.group_rows == 0) flush((up * 32) / p.group_rows, acc);
+    } else {
 #pragma unroll
-          for (int nt = 0; nt < NTK; nt++) {
-            const float tot = xhalf_sum(acc[nt]);
-            const int key = n0 + nt * 32 + r;
-            if (hh == 0 && key < p.Lk) csp[(int64_t)g * p.Lk + key] = tot;
-            acc[nt] = 0.f;
-          }
-        }
+      for (int ks = 0; ks < KS; ks++) {
+        if (ks + AHEAD < KS) frag[ks + AHEAD] = *(const bf16x8*)(qb + (kbase_l ^ ((ks + AHEAD) << 5)));
+        n0a = mfma32(frag[ks], kf[0][ks], n0a);
+        n1a = mfma32(frag[ks], kf[1][ks], n1a);
       }
     }
-    if (s + 1 < S) store_stage(st ^ 1);
+  };
+
+  // Tiles 0 .. U-2 go through the pipelined step (their successor exists); every tile whose rows are
+  // all valid is consumed inside the next step, the last tile (possibly ragged) by exp_acc below.
+  f32x16 sa0, sa1, sb0, sb1;
+  for (int s = 0; s < S; s++) {
+    if (s + 3 < S) issue_stage(s + 3);
+    const int u0 = 2 * s;
+    step(u0, sa0, sa1, sb0, sb1, u0 > 0);
+    if (u0 + 1 < U) step(u0 + 1, sb0, sb1, sa0, sa1, true);
+    wait_fills(min(s + 3, S - 1) - (s + 1));
     __syncthreads();
   }
+  // last tile U-1: in (sb) if U is even, else in (sa)
+  if (U & 1) exp_acc(U - 1, sa0, sa1); else exp_acc(U - 1, sb0, sb1);
+#endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int D, int NTK>
+template <int D>
 static int launch_cs(const ColsumParams& p0, hipStream_t stream) {
   ColsumParams p = p0;
-  p.nkt = (p.Lk + 4 * NTK * 32 - 1) / (4 * NTK * 32);
+  p.nkb = (p.Lk + 63) / 64;
+  p.nkt = (p.Lk + 255) / 256;
   p.total_wg = p.B * p.H * p.nkt;
   const int grid = ((p.total_wg + 7) / 8) * 8;
-  hipLaunchKernelGGL((colsum_kernel<D, NTK>), dim3(grid), dim3(256), 0, stream, p);
+  constexpr int SMEM = 4 * 64 * D * 2 + 8 * 256;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)colsum_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != hipSuccess)
+      return LVAR_ELAUNCH;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((colsum_kernel<D>), dim3(grid), dim3(256), SMEM, stream, p);
   return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
 }
 
 int launch_colsum(const ColsumParams& p, int head_dim, hipStream_t s) {
-  if (head_dim == 128) return launch_cs<128, 2>(p, s);
-  if (head_dim == 64) return launch_cs<64, 2>(p, s);
+  if (head_dim == 128) return launch_cs<128>(p, s);
+  if (head_dim == 64) return launch_cs<64>(p, s);
   return LVAR_EUNSUPPORTED;
 }
 

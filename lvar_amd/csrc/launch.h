@@ -13,7 +13,7 @@ struct AttnParams {
   const bf16_t *q, *k, *v;
   bf16_t* o;
   const bf16_t* o_accum;
-  float *M, *L;
+  float *M, *L, *LSE2;
   int64_t q_sb, q_sh, q_sr;
   int64_t k_sb, k_sh, k_sr;
   int64_t v_sb, v_sh, v_sr;
@@ -35,14 +35,15 @@ struct AttnParams {
 
 struct ColsumParams {
   const bf16_t *q, *k;
-  const float *M, *L;
+  const float* lse2;  // base-2 log-sum-exp per query row, M + log2(L)
   float* cs;
+  float* bs;          // optional per-64-key block sums [B,H,G,ceil(Lk/64)]
   int64_t q_sb, q_sh, q_sr;
   int64_t k_sb, k_sh, k_sr;
   int B, H, Lq, Lk, G;
   int group_rows;
   float c;
-  int nkt, total_wg;
+  int nkt, nkb, total_wg;
 };
 
 int launch_attn(const AttnParams& p, int head_dim, int mode, bool accum, bool lse_only, int nwaves, hipStream_t s);

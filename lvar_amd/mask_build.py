@@ -192,10 +192,18 @@ def key_block_sums(cs: torch.Tensor, block_k: int = 64) -> torch.Tensor:
     return F.pad(cs, (0, nb * block_k - Lk)).unflatten(-1, (nb, block_k)).sum(-1)
 
 
-def topk_block_lists(block_scores: torch.Tensor, keep_ratio: float) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Top ``round(keep_ratio*nK)`` key blocks per row (at least one), as sorted block lists."""
+def topk_block_lists(block_scores: torch.Tensor, keep_ratio: float, k_len: Optional[int] = None,
+                     block_k: int = 64) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Best-scoring key blocks per row as ascending block lists.  The number kept follows the
+    reference's token-count formula when ``k_len`` is given, ``block_k*round(keep_ratio*k_len/block_k)``
+    tokens = that many blocks (models/sparvar/sparse_attn.py:1012), else ``round(keep_ratio*nK)``;
+    at least one block is kept."""
     nK = block_scores.shape[-1]
-    k = max(1, min(nK, int(round(keep_ratio * nK))))
+    if k_len is not None:
+        k = indices_count(keep_ratio, k_len, block_k) // block_k
+    else:
+        k = int(round(keep_ratio * nK))
+    k = max(1, min(nK, k))
     idx = torch.topk(block_scores, k=k, dim=-1).indices.sort(-1).values.to(torch.int32)
     num = torch.full(block_scores.shape[:-1], k, dtype=torch.int32, device=block_scores.device)
     return num, idx.contiguous()

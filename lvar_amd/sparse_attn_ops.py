@@ -73,70 +73,75 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
+def _dense_launch(q, k, v, scale, want_o=True, want_ml=True, want_lse2=False):
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device) if want_o else None
+    M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device) if want_ml else None
+    L = torch.empty_like(M) if want_ml else None
+    lse2 = torch.empty((B, H, Lq), dtype=torch.float32, device=q.device) if want_lse2 else None
+    with torch.cuda.device(q.device):
+        st = _lib.load().lvar_dense_attn_fwd(_view(q), _view(k), _view(v if want_o else None), _view(o), _ptr(M), _ptr(L),
+                                            _ptr(lse2), B, H, Lq, Lk, d, _scale(q, scale), _stream(q))
+    _lib.check(st, "lvar_dense_attn_fwd")
+    return o, M, L, lse2
+
+
 def dense_attn(q, k, v, scale=None):
     """Dense flash attention, ``(o, (M, L))`` (reference ``dense_attn``, sparse_attn_ops.py:21-59,
     Triton-provider return convention: ``lse`` is the tuple ``(M, L)``, each ``[B,H,Lq,1]``)."""
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
     _check_qkv(q, k, v)
-    B, H, Lq, d = q.shape
-    Lk = k.shape[2]
-    o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device)
-    M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
-    L = torch.empty_like(M)
-    with torch.cuda.device(q.device):
-        st = _lib.load().lvar_dense_attn_fwd(_view(q), _view(k), _view(v), _view(o), M.data_ptr(), L.data_ptr(),
-                                            B, H, Lq, Lk, d, _scale(q, scale), _stream(q))
-    _lib.check(st, "lvar_dense_attn_fwd")
+    o, M, L, _ = _dense_launch(q, k, v, scale)
     return o, (M, L)
 
 
 def _lse_only(q, k, scale):
-    B, H, Lq, d = q.shape
-    M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
-    L = torch.empty_like(M)
-    with torch.cuda.device(q.device):
-        st = _lib.load().lvar_dense_attn_fwd(_view(q), _view(k), _view(None), _view(None), M.data_ptr(), L.data_ptr(),
-                                            B, H, Lq, k.shape[2], d, _scale(q, scale), _stream(q))
-    _lib.check(st, "lvar_dense_attn_fwd")
-    return M, L
+    """Statistics sweep without the PV product: base-2 log-sum-exp ``M + log2(L)``, fp32 [B,H,Lq]."""
+    return _dense_launch(q, k, None, scale, want_o=False, want_ml=False, want_lse2=True)[3]
 
 
-def _colsum_given_lse(q, k, M, L, scale, q_group_size):
+def _colsum_given_lse(q, k, lse2, scale, q_group_size, want_block_sums=False):
     B, H, Lq, d = q.shape
     Lk = k.shape[2]
     G = (Lq + q_group_size - 1) // q_group_size
     cs = torch.empty((B, H, G, Lk), dtype=torch.float32, device=q.device)
+    bs = torch.empty((B, H, G, (Lk + 63) // 64), dtype=torch.float32, device=q.device) if want_block_sums else None
     with torch.cuda.device(q.device):
-        st = _lib.load().lvar_colsum_fwd(_view(q), _view(k), M.data_ptr(), L.data_ptr(), cs.data_ptr(),
+        st = _lib.load().lvar_colsum_fwd(_view(q), _view(k), lse2.data_ptr(), cs.data_ptr(), _ptr(bs),
                                         B, H, Lq, Lk, d, q_group_size, _scale(q, scale), _stream(q))
     _lib.check(st, "lvar_colsum_fwd")
-    return cs
+    return (cs, bs) if want_block_sums else cs
 
 
-def colsum(q, k, scale=None, q_group_size: Optional[int] = None, lse: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
+def colsum(q, k, scale=None, q_group_size: Optional[int] = None, lse: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+           return_block_sums: bool = False):
     """Column sums of the softmax probabilities per group of ``q_group_size`` query rows
     (default: the kernel config's ``bm`` = 192), fp32 ``[B,H,G,Lk]``.  Self-contained two-pass form
-    (statistics sweep, then column sweep) unless ``lse=(M, L)`` from a previous dense pass is given."""
+    (statistics sweep, then column sweep) unless ``lse=(M, L)`` from a previous dense pass is given.
+    With ``return_block_sums`` also returns the sums over blocks of 64 keys, ``[B,H,G,ceil(Lk/64)]``."""
     q, k = _prep(q, "q"), _prep(k, "k")
     _check_qkv(q, k, k)
     if q_group_size is None:
         q_group_size = get_kernel_config_attn()["bm"]
     _require(q_group_size > 0 and q_group_size % 32 == 0, "q_group_size must be a positive multiple of 32")
     if lse is None:
-        M, L = _lse_only(q, k, scale)
+        lse2 = _lse_only(q, k, scale)
     else:
-        M, L = (t.to(torch.float32).contiguous() for t in lse)
+        M, L = lse
         _require(M.numel() == q.shape[0] * q.shape[1] * q.shape[2] == L.numel(), "lse must be ([B,H,Lq,1], [B,H,Lq,1])")
-    return _colsum_given_lse(q, k, M, L, scale, q_group_size)
+        lse2 = (M.to(torch.float32) + torch.log2(L.to(torch.float32))).reshape(q.shape[:3]).contiguous()
+    return _colsum_given_lse(q, k, lse2, scale, q_group_size, return_block_sums)
 
 
 def dense_colsum_attn(q, k, v, scale=None):
     """Kernel-level op ``(o, blocksums, (M, L))`` (reference Triton ``dense_colsum_attn``,
     kernels/sparse_attn/triton/attn_dense_colsum.py:237-296): dense attention, then the column
-    sweep that reuses its (M, L)."""
+    sweep that reuses its row statistics."""
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
-    o, (M, L) = dense_attn(q, k, v, scale)
-    cs = _colsum_given_lse(q, k, M, L, scale, get_kernel_config_attn()["bm"])
+    _check_qkv(q, k, v)
+    o, M, L, lse2 = _dense_launch(q, k, v, scale, want_lse2=True)
+    cs = _colsum_given_lse(q, k, lse2, scale, get_kernel_config_attn()["bm"])
     return o, cs, (M, L)
 
 

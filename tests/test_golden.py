@@ -78,10 +78,10 @@ def test_hip_matches_var_d16_fixture():
     bs = mb.key_block_sums(cs_all, 64)
     assert close(bs.cpu(), t(z["block_sums"]), 1e-5, 1e-3)
     # the mask derived from an identical colsum is bit-exact
-    num, idx = mb.topk_block_lists(t(z["block_sums"]).cuda(), 0.5)
+    num, idx = mb.topk_block_lists(t(z["block_sums"]).cuda(), 0.5, k_len=680)
     assert int(num[0, 0, 0]) == 5 and torch.equal(idx.cpu(), t(z["top5_blocks"]))
     # and here the HIP colsum ranks the same blocks (block sums differ by far more than its error)
-    num2, idx2 = mb.topk_block_lists(bs, 0.5)
+    num2, idx2 = mb.topk_block_lists(bs, 0.5, k_len=680)
     assert torch.equal(idx2.cpu(), t(z["top5_blocks"]))
     # block-sparse attention over those 5 blocks of 64 keys (one 128-row query block pair)
     nb = num2.expand(1, 1, 2).contiguous()

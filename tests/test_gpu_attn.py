@@ -87,6 +87,9 @@ def test_dense_attn_large_logits_rescale():
 
 
 COLSUM_SHAPES = [
+    (1, 2, 33, 25, 128),      # one ragged tile, fewer keys than a block
+    (1, 2, 4096, 300, 128),   # many stages: exercises the 4-deep LDS ring and its tail
+    (1, 1, 160, 64, 64),      # odd number of 32-row tiles
     (2, 16, 256, 680, 64),
     (1, 4, 256, 1000, 64),    # the reference's enabled self-test shape (attn_dense_colsum.py:573)
     (1, 2, 300, 1000, 128),   # last group has 108 rows
@@ -125,6 +128,13 @@ def test_colsum_standalone_groups_and_zero_query():
     assert torch.allclose(cs_all, ref_all, rtol=1e-3, atol=1e-6)
     assert torch.allclose(cs_192.sum(2, keepdim=True), cs_all, rtol=1e-4, atol=1e-6)
     assert torch.allclose(cs_32.sum(2, keepdim=True), cs_all, rtol=1e-4, atol=1e-6)
+    # fused per-64-key block sums (ragged last block: 680 = 10*64 + 40)
+    cs2, bs2 = ops.colsum(qg, kg, return_block_sums=True)
+    assert torch.equal(cs2.cpu(), cs_192) and bs2.shape == (B, H, 2, 11)
+    assert torch.allclose(bs2.cpu(), oracle.key_block_sums(cs_192, 64), rtol=1e-5, atol=1e-6)
+    # row statistics handed in from a previous dense pass give the same colsum
+    _, (M, L) = ops.dense_attn(qg, kg, dev(v)[0])
+    assert torch.allclose(ops.colsum(qg, kg, lse=(M, L)).cpu(), cs_192, rtol=1e-5, atol=1e-7)
     # q = 0  =>  uniform softmax  =>  cs = rows / Lk exactly representable up to rounding
     z = torch.zeros_like(qg)
     cs0 = ops.colsum(z, kg).cpu()

@@ -106,8 +106,9 @@ def test_block_lists_and_sums_match_oracle():
     assert torch.equal(oracle.lists_to_block_mask(n1, i1, 17), mask)
     cs = torch.rand(1, 2, 3, 680, generator=torch.Generator().manual_seed(4))
     assert torch.allclose(mb.key_block_sums(cs, 64), oracle.key_block_sums(cs, 64))
-    num, idx = mb.topk_block_lists(mb.key_block_sums(cs, 64), 0.5)
-    assert int(num[0, 0, 0]) == 6 or int(num[0, 0, 0]) == 5   # round(5.5) is half-to-even = 6
+    num, idx = mb.topk_block_lists(mb.key_block_sums(cs, 64), 0.5, k_len=680)
+    assert int(num[0, 0, 0]) == 5                              # 64*round(0.5*680/64)/64, BASELINE config 1
+    assert int(mb.topk_block_lists(mb.key_block_sums(cs, 64), 0.5)[0][0, 0, 0]) == 6   # round(5.5), half-to-even
     assert bool((idx[..., 1:] > idx[..., :-1]).all())
 
 
