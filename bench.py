@@ -162,8 +162,8 @@ def main():
         bq, bk = 128, (128 if wl == "video_10" else 64)
         nQ, nK = (Lq + bq - 1) // bq, (Lk + bk - 1) // bk
         if wl == "block_sparse_25":
-            cs = ops.colsum(qg, kg, scale, q_group_size=bq)                 # [B,H,nQ,Lk]
-            mask = mb.sink_window_topk_block_mask(mb.key_block_sums(cs, bk), bq, bk, density=0.25)
+            cs, bsum = ops.colsum(qg, kg, scale, q_group_size=bq, return_block_sums=True)   # [B,H,nQ,Lk], [B,H,nQ,nK]
+            mask = mb.sink_window_topk_block_mask(bsum, bq, bk, density=0.25)
             del cs
             config.update({"block": [bq, bk], "mask": "sink(scales<=16)+window(+-2 blocks/scale)+colsum top-k", "density": 0.25})
         elif wl == "video_10":
@@ -237,9 +237,14 @@ def main():
         cs_ms, _ = time_launches(lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 128), 10, 3)
         lse_ms, _ = time_launches(lambda: ops._lse_only(qg, kg, scale), 10, 3)
 
+        base = mb.sink_window_base_mask(128, 64, device=dev)
+        target = int(round(0.25 * base.shape[1]))
+
         def build():
             _, bs = ops._colsum_given_lse(qg, kg, lse2, scale, 128, want_block_sums=True)
-            return mb.block_mask_to_lists(mb.sink_window_topk_block_mask(bs, 128, 64, 0.25))
+            return ops.block_topk_lists(bs, target, base)
+        n2, i2 = build()
+        assert torch.equal(n2, num) and torch.equal(i2, idx), "GPU list build differs from the torch selection"
         build_ms, _ = time_launches(build, 5, 2)
         aux = {"dense_attn_ms": round(dense_ms, 4), "dense_attn_tflops": round(dense_flops / dense_ms / 1e9, 1),
                "colsum_given_lse_us": round(cs_ms * 1e3, 1), "lse_pass_us": round(lse_ms * 1e3, 1),

@@ -106,6 +106,22 @@ int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
                                int B, int H, int Lq, int Lk, int head_dim,
                                float scale, void* stream);
 
+/*
+ * Block-list build: for every (batch, head, query block) row of block_scores (fp32 contiguous
+ * [B,H,nQ,nK], e.g. the block sums of lvar_colsum_fwd with q_group_size = block_q) keep the blocks set
+ * in base_mask (uint8 [nQ,nK], shared by all batches and heads, may be NULL) plus the best-scoring
+ * other blocks until `target` blocks are kept (all base blocks are kept even beyond target), and
+ * write the ascending compacted list: kv_num_blocks int32 [B,H,nQ], kv_indices int32 [B,H,nQ,nK]
+ * (unused tail zero).  Ties go to the smaller block index (stable descending order), so the lists are
+ * a pure function of the scores.  nK <= 2048.
+ * Does on the GPU what the reference does with torch.topk plus list padding
+ * (models/sparvar/sparse_attn.py:1012-1036) and what its unused mask_to_indices / topk_indices
+ * helpers compact (kernels/chipmunk/csrc/indexed_io/mask_to_indices.cu:21-97, topk_indices.cu:26-145).
+ */
+int lvar_block_topk_lists(const float* block_scores, const uint8_t* base_mask,
+                          int32_t* kv_num_blocks, int32_t* kv_indices,
+                          int B, int H, int nQ, int nK, int target, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,6 +13,7 @@ from .build import LIB_PATH
 EXPORTED_SYMBOLS = (
     "lvar_version", "lvar_target_arch", "lvar_status_string",
     "lvar_dense_attn_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_block_sparse_attn_fwd",
+    "lvar_block_topk_lists",
 )
 
 
@@ -54,6 +55,8 @@ def load() -> C.CDLL:
     lib.lvar_csp_attn_fwd.argtypes = [T, T, T, T, T, P, P, P, P, I, I64, I, I, I, I, I, I, F, F, P]
     lib.lvar_block_sparse_attn_fwd.restype = I
     lib.lvar_block_sparse_attn_fwd.argtypes = [T, T, T, T, P, P, P, I64, I64, P, I64, I64, I64, I, I, I, I, I, I, I, I, F, P]
+    lib.lvar_block_topk_lists.restype = I
+    lib.lvar_block_topk_lists.argtypes = [P, P, P, P, I, I, I, I, I, P]
     _lib = lib
     return lib
 

@@ -145,4 +145,14 @@ int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
   return launch_attn(p, head_dim, MODE_BLOCK, false, false, 4, (hipStream_t)stream);
 }
 
+int lvar_block_topk_lists(const float* block_scores, const uint8_t* base_mask, int32_t* kv_num_blocks,
+                          int32_t* kv_indices, int B, int H, int nQ, int nK, int target, void* stream) {
+  if (!block_scores || !kv_num_blocks || !kv_indices || B <= 0 || H <= 0 || nQ <= 0 || nK <= 0 || target < 0)
+    return LVAR_EINVAL;
+  MaskListParams p{};
+  p.scores = block_scores; p.base = base_mask; p.kv_num_blocks = kv_num_blocks; p.kv_indices = kv_indices;
+  p.rows = B * H * nQ; p.nQ = nQ; p.nK = nK; p.target = target;
+  return launch_block_topk_lists(p, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -46,6 +46,15 @@ struct ColsumParams {
   int nkt, nkb, total_wg;
 };
 
+struct MaskListParams {
+  const float* scores;     // [rows, nK]
+  const uint8_t* base;     // [nQ, nK] or null
+  int32_t* kv_num_blocks;  // [rows]
+  int32_t* kv_indices;     // [rows, nK]
+  int rows, nQ, nK, target;
+};
+
+int launch_block_topk_lists(const MaskListParams& p, hipStream_t s);
 int launch_attn(const AttnParams& p, int head_dim, int mode, bool accum, bool lse_only, int nwaves, hipStream_t s);
 int launch_colsum(const ColsumParams& p, int head_dim, hipStream_t s);
 

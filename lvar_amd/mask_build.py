@@ -20,7 +20,7 @@ INFINITY_SCALES = (1, 2, 4, 6, 8, 12, 16, 20, 24, 32, 40, 48, 64)
 __all__ = [
     "INFINITY_SCALES", "scale_offsets", "indices_count", "topk_index_list", "map_inds_counts_across_scales",
     "local_group_runs", "append_local_run", "upsample_ocache", "flex_block_mask", "block_mask_to_lists",
-    "key_block_sums", "topk_block_lists", "sink_window_topk_block_mask",
+    "key_block_sums", "topk_block_lists", "sink_window_base_mask", "sink_window_topk_block_mask",
 ]
 
 
@@ -209,23 +209,20 @@ def topk_block_lists(block_scores: torch.Tensor, keep_ratio: float, k_len: Optio
     return num, idx.contiguous()
 
 
-def sink_window_topk_block_mask(block_scores: torch.Tensor, block_q: int = 128, block_k: int = 64, density: float = 0.25,
-                                sink_scale: int = 7, window: int = 2, scales: Sequence[int] = INFINITY_SCALES) -> torch.Tensor:
-    """Block mask of the Infinity last-scale benchmark configuration: all key blocks of scales
-    below ``sink_scale`` (keys < 521), +-``window`` key blocks around the query block's position
-    rescaled into every later scale, then the best-scoring remaining blocks by ``block_scores``
-    [B,H,nQ,nK] (colsum summed per query block and key block) up to ``round(density*nK)`` per row."""
+def sink_window_base_mask(block_q: int = 128, block_k: int = 64, sink_scale: int = 7, window: int = 2,
+                          scales: Sequence[int] = INFINITY_SCALES, device=None) -> torch.Tensor:
+    """Score-independent part of the Infinity last-scale benchmark mask, bool [nQ, nK]: all key blocks
+    of scales below ``sink_scale`` (keys < 521 for 7) and, in every later scale, +-``window`` key blocks
+    around the query block's centre rescaled into that scale's grid."""
     offs = scale_offsets(scales)
     Hq = scales[-1]
     Sq, Sk = Hq * Hq, offs[-1]
     nQ, nK = (Sq + block_q - 1) // block_q, (Sk + block_k - 1) // block_k
-    dev = block_scores.device
-    assert tuple(block_scores.shape[2:]) == (nQ, nK), (tuple(block_scores.shape), nQ, nK)
-    base = torch.zeros(nQ, nK, dtype=torch.bool, device=dev)
+    base = torch.zeros(nQ, nK, dtype=torch.bool, device=device)
     base[:, :(offs[sink_scale] + block_k - 1) // block_k] = True
-    qc = torch.clamp(torch.arange(nQ, device=dev) * block_q + block_q // 2, max=Sq - 1)
+    qc = torch.clamp(torch.arange(nQ, device=device) * block_q + block_q // 2, max=Sq - 1)
     qy, qx = qc // Hq, qc % Hq
-    cols = torch.arange(nK, device=dev)[None, :]
+    cols = torch.arange(nK, device=device)[None, :]
     for si in range(sink_scale, len(scales)):
         Hk = scales[si]
         ky = torch.clamp(qy * Hk // Hq, max=Hk - 1)
@@ -234,6 +231,18 @@ def sink_window_topk_block_mask(block_scores: torch.Tensor, block_q: int = 128, 
         lo = torch.clamp(j - window, min=offs[si] // block_k)[:, None]
         hi = torch.clamp(j + window, max=(offs[si + 1] - 1) // block_k)[:, None]
         base |= (cols >= lo) & (cols <= hi)
+    return base
+
+
+def sink_window_topk_block_mask(block_scores: torch.Tensor, block_q: int = 128, block_k: int = 64, density: float = 0.25,
+                                sink_scale: int = 7, window: int = 2, scales: Sequence[int] = INFINITY_SCALES) -> torch.Tensor:
+    """Block mask of the Infinity last-scale benchmark configuration: :func:`sink_window_base_mask`,
+    then the best-scoring remaining blocks by ``block_scores`` [B,H,nQ,nK] (colsum summed per query
+    block and key block) up to ``round(density*nK)`` per row; ties go to the smaller block index.
+    (The same selection runs on the GPU in ``sparse_attn_ops.block_topk_lists``.)"""
+    base = sink_window_base_mask(block_q, block_k, sink_scale, window, scales, block_scores.device)
+    nQ, nK = base.shape
+    assert tuple(block_scores.shape[2:]) == (nQ, nK), (tuple(block_scores.shape), nQ, nK)
     target = int(round(density * nK))
     extra = (target - base.sum(-1)).clamp(min=0)                               # [nQ]
     score = block_scores.to(torch.float32).masked_fill(base, -float("inf"))

@@ -23,7 +23,7 @@ from .sparse_attn_config import get_kernel_config_attn
 
 __all__ = [
     "dense_attn", "dense_colsum_attn", "dense_colsum_attn_s", "dense_colsum_attn_q", "colsum",
-    "csp_attn", "csp_attn_delta", "block_sparse_attn", "ShapeError",
+    "csp_attn", "csp_attn_delta", "block_sparse_attn", "block_topk_lists", "ShapeError",
 ]
 
 
@@ -248,3 +248,27 @@ def block_sparse_attn(q, k, v, kv_num_blocks, kv_indices, block_q: int = 128, bl
             block_q, block_k, B, H, Lq, Lk, d, _scale(q, scale), _stream(q))
     _lib.check(st, "lvar_block_sparse_attn_fwd")
     return o, (M, L)
+
+
+def block_topk_lists(block_scores, target: int, base_mask=None):
+    """Block lists from block scores on the GPU: per ``[B,H,nQ]`` row keep the blocks of ``base_mask``
+    (bool/uint8 ``[nQ,nK]``, optional) plus the best-scoring others up to ``target`` blocks; returns
+    ``(kv_num_blocks int32 [B,H,nQ], kv_indices int32 [B,H,nQ,nK])`` in ascending block order with a
+    zero tail, ready for :func:`block_sparse_attn`.  Ties go to the smaller block index."""
+    _require(block_scores.dim() == 4, "block_scores must be [B,H,nQ,nK]")
+    if not block_scores.is_cuda:
+        raise RuntimeError("block_scores must live on a HIP device; lvar_amd has no CPU path")
+    bs = block_scores.to(torch.float32).contiguous()
+    B, H, nQ, nK = bs.shape
+    _require(nK <= 2048, "at most 2048 key blocks per row")
+    base = None
+    if base_mask is not None:
+        _require(tuple(base_mask.shape) == (nQ, nK), f"base_mask must be [nQ,nK] = {(nQ, nK)}")
+        base = base_mask.to(device=bs.device, dtype=torch.uint8).contiguous()
+    num = torch.empty((B, H, nQ), dtype=torch.int32, device=bs.device)
+    idx = torch.empty((B, H, nQ, nK), dtype=torch.int32, device=bs.device)
+    with torch.cuda.device(bs.device):
+        st = _lib.load().lvar_block_topk_lists(bs.data_ptr(), _ptr(base), num.data_ptr(), idx.data_ptr(),
+                                              B, H, nQ, nK, int(target), _stream(bs))
+    _lib.check(st, "lvar_block_topk_lists")
+    return num, idx

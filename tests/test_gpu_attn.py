@@ -265,6 +265,36 @@ def test_block_sparse_full_mask_equals_dense_and_broadcast():
     assert torch.equal(o0[:, :, 128:], od[:, :, 128:])
 
 
+def test_block_topk_lists_bit_exact():
+    """The GPU list build is a pure function of the scores: identical to the torch selection."""
+    from lvar_amd import mask_build as mb
+    from lvar_amd import sparse_attn_ops as ops
+    g = torch.Generator().manual_seed(0)
+    scores = torch.rand(2, 3, 32, 165, generator=g)
+    scores[0, 0, 3, 20:60] = 0.5                       # ties: smaller block index wins
+    base = mb.sink_window_base_mask()
+    target = round(0.25 * 165)
+    num, idx = ops.block_topk_lists(scores.cuda(), target, base)
+    n_ref, i_ref = mb.block_mask_to_lists(mb.sink_window_topk_block_mask(scores))
+    assert torch.equal(num.cpu(), n_ref) and torch.equal(idx.cpu(), i_ref)
+    assert bool((num == target).all())
+    # no base mask, plain top-k; target larger than the row keeps everything; target 0 keeps nothing
+    s2 = torch.rand(1, 2, 5, 70, generator=g)
+    num, idx = ops.block_topk_lists(s2.cuda(), 7)
+    n_ref, i_ref = mb.topk_block_lists(s2, 0.1)
+    assert int(n_ref[0, 0, 0]) == 7 and torch.equal(num.cpu(), n_ref) and torch.equal(idx.cpu()[..., :7], i_ref)
+    assert bool((idx.cpu()[..., 7:] == 0).all())
+    num, idx = ops.block_topk_lists(s2.cuda(), 500)
+    assert bool((num == 70).all()) and torch.equal(idx.cpu()[0, 0, 0], torch.arange(70, dtype=torch.int32))
+    num, idx = ops.block_topk_lists(s2.cuda(), 0)
+    assert bool((num == 0).all()) and bool((idx == 0).all())
+    # base blocks are kept even when they exceed the target
+    b2 = torch.zeros(5, 70, dtype=torch.bool)
+    b2[:, :10] = True
+    num, idx = ops.block_topk_lists(s2.cuda(), 4, b2)
+    assert bool((num == 10).all()) and torch.equal(idx.cpu()[0, 1, 2, :10], torch.arange(10, dtype=torch.int32))
+
+
 def test_errors():
     from lvar_amd import sparse_attn_ops as ops
     q, k, v = make_qkv(1, 1, 64, 64, 128, seed=1)
