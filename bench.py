@@ -117,7 +117,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="block_sparse_25",
-                    help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | density_<pct> | video_10")
+                    help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | density_<pct> | video_10 | copy_1gib")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aux", action="store_true", help="skip the companion dense/colsum/mask-build timings")
     ap.add_argument("--cpu-budget-s", type=float, default=20.0)
@@ -137,6 +137,15 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     wl = args.workload
+    if wl == "copy_1gib":
+        # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
+        x = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+        y = torch.empty_like(x)
+        ms, _ = time_launches(lambda: y.copy_(x), args.steps, args.warmup)
+        print(json.dumps({"metric": "device copy bandwidth", "value": round(2 * x.numel() * 4 / ms / 1e6, 1), "unit": "GB/s",
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+                          "config": {"workload": wl, "bytes_read": x.numel() * 4, "bytes_written": x.numel() * 4}}))
+        return
     d = 128
     aux = {}
     cpu = None
@@ -192,14 +201,14 @@ def main():
         flops = block_flops(num, idx, Lq, Lk, d, bq, bk, B, H)
         config["active_block_fraction"] = round(float(mask.float().mean().item()), 4)
         fn = lambda: ops.block_sparse_attn(qg, kg, vg, num, idx, bq, bk, scale)
-        kernel = "attn_fwd_kernel<128,4,BLOCK>"
+        kernel = "attn_fwd_kernel<128,4,MODE_BLOCK>"
         if not args.no_cpu_baseline:
             val, sample = cpu_baseline_block_sparse(q, k, v, num.cpu(), idx.cpu(), bq, bk, args.cpu_budget_s)
             cpu = {"value": round(val, 5), "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port", "sample": sample}
     elif wl == "dense":
         flops = dense_flops
         fn = lambda: ops.dense_attn(qg, kg, vg, scale)
-        kernel = "attn_fwd_kernel<128,4,DENSE>"
+        kernel = "attn_fwd_kernel<128,4,MODE_BLOCK> (identity list)"
         if not args.no_cpu_baseline:
             done, t = cpu_baseline_dense(q, k, v, args.cpu_budget_s)
             cpu = {"value": round(dense_flops / (B * H) * done / t / 1e12, 5), "unit": "TFLOP/s", "cores": os.cpu_count(),
@@ -224,7 +233,7 @@ def main():
         flops = 4.0 * d * B * H * float(rows.sum()) * cnt
         o0 = torch.zeros_like(qg)
         fn = lambda: ops.csp_attn(qg, kg, vg, scale, inds, counts, o0, 1)
-        kernel = "attn_fwd_kernel<128,6,GATHER>"
+        kernel = "attn_fwd_kernel<128,6,MODE_GATHER>"
         config.update({"top_keys": 0.2, "count": cnt})
 
     ms, wall_ms = time_launches(fn, args.steps, args.warmup)
@@ -251,7 +260,8 @@ def main():
                "colsum_plus_mask_build_ms": round(build_ms, 4), "speedup_vs_dense": round(dense_ms / ms, 3)}
 
     out = {
-        "metric": "block-sparse attn effective TFLOP/s over active blocks" if kernel.endswith("BLOCK>") else f"{wl} effective TFLOP/s",
+        "metric": ("block-sparse attn effective TFLOP/s (% bf16 MFMA peak); colsum us @Infinity-2B 1024^2"
+                   if wl == "block_sparse_25" else f"{wl} effective TFLOP/s"),
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic (seeded N(0,1)*%.1f, random-init, no checkpoint)" % amp,
