@@ -142,29 +142,38 @@ def upsample_ocache(o_cache: torch.Tensor, L_src: int, L_tgt: int) -> torch.Tens
     return x.view(B, H, Dh, ht, ht).permute(0, 1, 3, 4, 2).reshape(B, H, ht * ht, Dh)
 
 
+def _hw(scales) -> List[Tuple[int, int]]:
+    return [(int(s), int(s)) if isinstance(s, int) else (int(s[0]), int(s[1])) for s in scales]
+
+
 def flex_block_mask(q_scale_idx: int, kernel_schedule: Sequence[int], attn_sink_scale: int, block_size: int = 128,
-                    block_k: Optional[int] = None, scales: Sequence[int] = INFINITY_SCALES, device=None) -> torch.Tensor:
+                    block_k: Optional[int] = None, scales: Sequence = INFINITY_SCALES, device=None) -> torch.Tensor:
     """Attention-sink + local-window block mask of ``SparseFlexAttn``
     (models/sparvar/basic_sparvar.py:74-185): a key is attended if it lies below
     ``cum[attn_sink_scale]`` or inside the square window (per-key-scale kernel size, negative =
     never) around the query position rescaled to the key's grid; a block is kept if any of its
-    elements is.  Returns bool [nQ, nK] for (block_size x block_k) blocks."""
+    elements is.  ``scales`` holds side lengths or ``(h, w)`` pairs (the reference's
+    ``scale_schedule``).  Returns bool [nQ, nK] for (block_size x block_k) blocks."""
     bq, bk = block_size, (block_size if block_k is None else block_k)
-    offs = scale_offsets(scales)
-    Hq = scales[q_scale_idx]
-    Sq, Sk = Hq * Hq, offs[q_scale_idx + 1]
+    hw = _hw(scales)[:q_scale_idx + 1]
+    offs = [0]
+    for h_, w_ in hw:
+        offs.append(offs[-1] + h_ * w_)
+    Hq, Wq = hw[q_scale_idx]
+    Sq, Sk = Hq * Wq, offs[-1]
     sink = offs[attn_sink_scale] if attn_sink_scale > 0 else 0
     kv = torch.arange(Sk, device=device)
-    bounds = torch.tensor(offs[:q_scale_idx + 2], device=device)
+    bounds = torch.tensor(offs, device=device)
     si = torch.searchsorted(bounds, kv, right=True) - 1
-    Hk = torch.tensor(list(scales[:q_scale_idx + 1]), device=device)[si]
+    Hk = torch.tensor([h_ for h_, _ in hw], device=device)[si]
+    Wk = torch.tensor([w_ for _, w_ in hw], device=device)[si]
     ksz = torch.tensor(list(kernel_schedule[:q_scale_idx + 1]), device=device)[si]
     rel = kv - bounds[si]
-    ky, kx = rel // Hk, rel % Hk
+    ky, kx = rel // Wk, rel % Wk
     qi = torch.arange(Sq, device=device)
-    qy, qx = (qi // Hq).float(), (qi % Hq).float()
+    qy, qx = (qi // Wq).float(), (qi % Wq).float()
     cy = torch.round((qy / Hq)[:, None] * Hk[None, :])
-    cx = torch.round((qx / Hq)[:, None] * Hk[None, :])
+    cx = torch.round((qx / Wq)[:, None] * Wk[None, :])
     half = torch.div(ksz, 2, rounding_mode="floor")[None, :]
     fine = ((cy - ky[None, :]).abs() <= half) & ((cx - kx[None, :]).abs() <= half)
     fine |= (kv < sink)[None, :]

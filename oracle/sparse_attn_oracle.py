@@ -344,33 +344,34 @@ def flex_block_mask(q_scale_idx, kernel_schedule, attn_sink_scale, block_size=12
     """CSLA block mask (models/sparvar/basic_sparvar.py:74-185) by brute force over (q, kv):
     sink ``kv < cum[attn_sink_scale]`` OR a per-key-scale square window around the rescaled
     query position (``round(qy/Hq*Hk)`` computed in float32, half-to-even), negative kernel
-    size => never attended; then ``any`` over block tiles.  Returns bool [nQ, nK]."""
+    size => never attended; then ``any`` over block tiles.  ``scales``: side lengths or (h, w) pairs.
+    Returns bool [nQ, nK]."""
     bq = block_size
     bk = block_size if block_k is None else block_k
-    cum = infinity_cum(scales)
-    Hq = scales[q_scale_idx]
-    Sq, Sk = Hq * Hq, cum[q_scale_idx + 1]
+    hw = [(s, s) if isinstance(s, int) else (s[0], s[1]) for s in scales]
+    cum = [0]
+    for h_, w_ in hw:
+        cum.append(cum[-1] + h_ * w_)
+    Hq, Wq = hw[q_scale_idx]
+    Sq, Sk = Hq * Wq, cum[q_scale_idx + 1]
     sink = cum[attn_sink_scale] if attn_sink_scale > 0 else 0
     nQ, nK = (Sq + bq - 1) // bq, (Sk + bk - 1) // bk
     mask = np.zeros((nQ, nK), dtype=bool)
-    kv_scale = np.zeros(Sk, dtype=np.int64)
     for si in range(q_scale_idx + 1):
-        kv_scale[cum[si]:cum[si + 1]] = si
-    for kv in range(Sk):
-        si = kv_scale[kv]
-        Hk = scales[si]
-        rel = kv - cum[si]
-        ky, kx = rel // Hk, rel % Hk
+        Hk, Wk = hw[si]
         half = kernel_schedule[si] // 2  # python floor division: -1 // 2 == -1
-        for qi in range(Sq):
-            hit = kv < sink
-            if not hit:
-                qy, qx = qi // Hq, qi % Hq
-                cy = np.rint(np.float32(np.float32(qy) / np.float32(Hq)) * np.float32(Hk))
-                cx = np.rint(np.float32(np.float32(qx) / np.float32(Hq)) * np.float32(Hk))
-                hit = abs(cy - ky) <= half and abs(cx - kx) <= half
-            if hit:
-                mask[qi // bq, kv // bk] = True
+        for kv in range(cum[si], cum[si + 1]):
+            rel = kv - cum[si]
+            ky, kx = rel // Wk, rel % Wk
+            for qi in range(Sq):
+                hit = kv < sink
+                if not hit:
+                    qy, qx = qi // Wq, qi % Wq
+                    cy = np.rint(np.float32(np.float32(qy) / np.float32(Hq)) * np.float32(Hk))
+                    cx = np.rint(np.float32(np.float32(qx) / np.float32(Wq)) * np.float32(Wk))
+                    hit = abs(cy - ky) <= half and abs(cx - kx) <= half
+                if hit:
+                    mask[qi // bq, kv // bk] = True
     return torch.from_numpy(mask)
 
 

@@ -1,0 +1,104 @@
+"""The caller-level mirrors (SparseFlexAttn, SparseDiffAttn, torch.ops.lvar.*) on the GPU against
+compositions of oracle functions on the same seeded inputs."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from conftest import make_qkv
+
+pytestmark = pytest.mark.gpu
+
+SCALES9 = (1, 2, 4, 6, 8, 12, 16, 20, 24)   # Infinity's first nine scales: a small but real schedule
+
+
+def close(a, b, atol=2e-2, rtol=1e-2):
+    return bool(((a.float().cpu() - b).abs() <= atol + rtol * b.abs()).all())
+
+
+def test_sparse_flex_attn_matches_oracle():
+    from lvar_amd.sparse_flex_attn import SparseFlexAttn
+    ks = [-1, -1, -1, -1, 1, 1, 3, 5, 7]
+    mod = SparseFlexAttn([(s, s) for s in SCALES9], ks, q_scale_idx=8, attn_sink_scale=3, num_heads=2)
+    mask = oracle.flex_block_mask(8, ks, 3, 128, scales=SCALES9)
+    assert torch.equal(mod.block_level_mask, mask)
+    q, k, v = make_qkv(2, 2, 576, 1497, 128, seed=8, amp=0.5)
+    num, idx = oracle.block_mask_to_lists(mask.expand(2, 2, *mask.shape))
+    ref, _, _ = oracle.block_sparse_attn(q, k, v, num, idx, 128, 128, scale=1.0)
+    # cosine-attention callers hand q, k in fp32 and v in bf16 (basic_sparvar.py:362-367)
+    out = mod(q.float().cuda(), k.float().cuda(), v.cuda(), scale=1.0)
+    assert out.dtype == torch.bfloat16 and close(out, ref)
+    with pytest.raises(ValueError):
+        mod(q[:, :, :100].cuda(), k.cuda(), v.cuda())
+
+
+def test_sparse_diff_attn_full_and_sparse_steps():
+    from lvar_amd import sparse_attn_config as cfg
+    from lvar_amd.sparse_diff_attn import SparseDiffAttn
+    cfg.reset()
+    cfg.GLOBAL_CONFIG["attn"]["top_keys"] = 0.25
+    try:
+        mod = SparseDiffAttn(scales=SCALES9, spsd_scale=6)
+        cum = oracle.infinity_cum(SCALES9)
+        B, H, d = 1, 2, 128
+        g = torch.Generator().manual_seed(3)
+        mk = lambda L: (torch.randn(B, H, L, d, generator=g) * 0.5).to(torch.bfloat16)
+        # --- full step at the decision scale (16x16 queries, 521 keys) ---
+        q, k, v = mk(256), mk(cum[7]), mk(cum[7])
+        o = mod(q.cuda(), k.cuda(), v.cuda(), None, do_full_step=True, scale_ind=6)
+        o_ref, cs_ref, _ = oracle.dense_colsum_attn(q, k, v)
+        assert close(o, o_ref)
+        cnt = oracle.indices_count(0.25, cum[7], 64)
+        assert cnt == 128 and int(mod.counts[0, 0, 0]) == cnt and mod.indices.shape == (B, H, 2, cum[7])
+        # the lists are the top-k of the HIP colsum; the oracle's top-k set agrees wherever the k-th
+        # value is separated by more than the colsum tolerance
+        sel = mod.indices[..., :cnt].cpu().long()
+        picked = torch.gather(cs_ref, -1, sel)
+        kth = torch.topk(cs_ref, cnt, dim=-1).values[..., -1:]
+        assert bool((picked >= kth * (1 - 2e-3)).all())
+        cache_ref = oracle.csp_attn(q, k, v, None, mod.indices.cpu(), mod.counts.cpu(), o.cpu(), -1)
+        assert close(mod.out_cache, cache_ref)
+        # --- sparse steps at the next two scales ---
+        for si in (7, 8):
+            S = SCALES9[si]
+            inds_prev, counts_prev, cache_prev = mod.indices.cpu(), mod.counts.cpu(), mod.out_cache.cpu()
+            q, k, v = mk(S * S), mk(cum[si + 1]), mk(cum[si + 1])
+            out = mod(q.cuda(), k.cuda(), v.cuda(), None, scale_ind=si)
+            mi, mc = oracle.map_inds_counts_across_scales(inds_prev, counts_prev, S * S, cum[si + 1])
+            ia, kv = oracle.crossscale_self_indices(si, cfg.GLOBAL_CONFIG["attn"]["cs4a_ws"][-(9 - si)], SCALES9)
+            runs, L = oracle.aggregate_group_indices(ia, S * S, kv, 192, 64)
+            G = mi.shape[2]
+            full = torch.zeros(B, H, G, cum[si + 1], dtype=torch.int32)
+            full[..., :mi.shape[-1]] = mi
+            full[..., mi.shape[-1]:mi.shape[-1] + L] = runs.to(torch.int32)
+            counts = torch.full((B, H, G), mi.shape[-1] + L, dtype=torch.int32)
+            up = oracle.upsample_ocache(cache_prev.float(), cache_prev.shape[-2], S * S).to(torch.bfloat16)
+            ref = oracle.csp_attn(q, k, v, None, full, counts, up, 1)
+            assert close(out, ref, atol=3e-2), si
+            if si == 7:
+                assert torch.equal(mod.indices.cpu()[..., :int(counts[0, 0, 0])], full[..., :int(counts[0, 0, 0])])
+    finally:
+        cfg.reset()
+
+
+def test_torch_ops_chipmunk_schemas():
+    import lvar_amd.torch_ops  # noqa: F401
+    q, k, v = make_qkv(1, 2, 384, 500, 128, seed=12, amp=0.3)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    o, lse = torch.ops.lvar.dense_attn(qg, kg, vg)
+    o_ref, M, L = oracle.dense_attn(q, k, v, scale=1.0)
+    assert close(o, o_ref) and lse.shape == (1, 2, 384, 1)
+    # the reference's constant: 1 / (2^M * L)  (dense_attn.cu:227-230)
+    assert torch.allclose(lse.cpu(), 1.0 / (torch.exp2(M) * L), rtol=2e-3)
+    o2, cs, l = torch.ops.lvar.dense_colsum_attn(qg, kg, vg, lse)
+    _, cs_ref, _ = oracle.dense_colsum_attn(q, k, v, scale=1.0)
+    assert torch.equal(o2, o) and torch.allclose(cs.cpu(), cs_ref, rtol=2e-3, atol=1e-6) and torch.allclose(l, lse)
+    inds = torch.arange(500, dtype=torch.int32).flip(0).expand(1, 2, 2, 500).contiguous()
+    counts = torch.full((1, 2, 2), 192, dtype=torch.int32)
+    oc = o.clone()
+    assert torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds.cuda(), counts.cuda(), -1) is None
+    ref = oracle.csp_attn(q, k, v, 1.0, inds, counts, o.cpu(), -1)
+    assert close(oc, ref) and not torch.equal(oc, o)
+    with pytest.raises(Exception):
+        torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds.cuda(), counts.cuda(), 2)
