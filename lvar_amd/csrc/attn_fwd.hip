@@ -298,13 +298,8 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     auto body = [&](int t, auto par, auto masked, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1) {
       constexpr int PAR = decltype(par)::value;
       constexpr bool MASKED = decltype(masked)::value;
-#ifdef LVAR_K_FIRST
-      if (t + 2 < T) issue(krsrc, k_srb, false, rows_k, lds0 + PAR * TILE);
-      if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows_v, lds0 + (3 - PAR) * TILE);
-#else
       if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows_v, lds0 + (3 - PAR) * TILE);
       if (t + 2 < T) issue(krsrc, k_srb, false, rows_k, lds0 + PAR * TILE);
-#endif
       if (t + 3 < T) finish_rows(t + 3, raw, rows_n, nv3);
       if (t + 4 < T) prefetch_raw(t + 4, raw);
       // The block below is software-pipelined by hand; sched_barrier(0) after every step stops the
@@ -333,20 +328,11 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
 #pragma unroll
       for (int j = 0; j < AHEAD; j++) frag[j] = kread(j);
       __builtin_amdgcn_sched_barrier(0);
-#ifdef LVAR_SETPRIO
-      __builtin_amdgcn_s_setprio(LVAR_SETPRIO);
-#endif
 #pragma unroll
       for (int j = 0; j < NQK; j++) {
-#ifdef LVAR_EXP_HALFREADS  // experiment only (wrong results): every second K fragment read is skipped
-        if (j + AHEAD < NQK && !((j + AHEAD) & 1)) frag[j + AHEAD] = kread(j + AHEAD);
-        if (j & 1) n1 = mfma32(frag[j & ~1], qf[j >> 1], n1);
-        else n0 = mfma32(frag[j], qf[j >> 1], n0);
-#else
         if (j + AHEAD < NQK) frag[j + AHEAD] = kread(j + AHEAD);
         if (j & 1) n1 = mfma32(frag[j], qf[j >> 1], n1);
         else n0 = mfma32(frag[j], qf[j >> 1], n0);
-#endif
         // exp2 share of this step: 32 / NQK element pairs of S(t)
 #pragma unroll
         for (int u = 0; u < 16 / NQK; u++) {
@@ -376,13 +362,8 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
         if (MASKED) mask_tile(n0, n1, nv1);
 #pragma unroll
         for (int j = 0; j < NPV; j++) {
-#ifdef LVAR_EXP_HALFREADS
-          if (j + AHEAD < NPV && !((j + AHEAD) & 1)) frag[j + AHEAD] = vread(j + AHEAD);
-          oacc[j % MTD] = mfma32(frag[j & ~1], pb[j / MTD], oacc[j % MTD]);
-#else
           if (j + AHEAD < NPV) frag[j + AHEAD] = vread(j + AHEAD);
           oacc[j % MTD] = mfma32(frag[j], pb[j / MTD], oacc[j % MTD]);
-#endif
           // row-maximum share: spread the 32 elements of S(t+1) over the steps after the first AHEAD
           constexpr int MSTEPS = NPV - AHEAD;
           if (j >= AHEAD) {
@@ -400,9 +381,6 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
         for (int e = 0; e < 16; e++) ma = fmaxf(fmaxf(ma, n0[e]), n1[e]);
       }
       const float mx = xhalf_max(fmaxf(ma, mb));
-#ifdef LVAR_SETPRIO
-      __builtin_amdgcn_s_setprio(0);
-#endif
       __builtin_amdgcn_s_waitcnt(0x0f70);
       __syncthreads();
       rescale_check(mx);
