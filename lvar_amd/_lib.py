@@ -13,7 +13,7 @@ from .build import LIB_PATH
 EXPORTED_SYMBOLS = (
     "lvar_version", "lvar_target_arch", "lvar_status_string",
     "lvar_dense_attn_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_block_sparse_attn_fwd",
-    "lvar_block_topk_lists",
+    "lvar_block_topk_lists", "lvar_topk_token_lists", "lvar_remap_concat_lists", "lvar_mask_to_lists",
 )
 
 
@@ -57,6 +57,12 @@ def load() -> C.CDLL:
     lib.lvar_block_sparse_attn_fwd.argtypes = [T, T, T, T, P, P, P, I64, I64, P, I64, I64, I64, I, I, I, I, I, I, I, I, F, P]
     lib.lvar_block_topk_lists.restype = I
     lib.lvar_block_topk_lists.argtypes = [P, P, P, P, I, I, I, I, I, P]
+    lib.lvar_topk_token_lists.restype = I
+    lib.lvar_topk_token_lists.argtypes = [P, I64, P, I64, P, I, I, I, P]
+    lib.lvar_remap_concat_lists.restype = I
+    lib.lvar_remap_concat_lists.argtypes = [P, I64, I, P, I64, I, P, I64, P, I, I, I, I, I, P]
+    lib.lvar_mask_to_lists.restype = I
+    lib.lvar_mask_to_lists.argtypes = [P, I64, P, I64, P, I, I, I, P]
     _lib = lib
     return lib
 

@@ -69,6 +69,13 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const int bh = w / p.nqt, qt = w - bh * p.nqt;
   const int b = bh / p.H, h = bh - b * p.H;
   const int tid = threadIdx.x, lane = tid & 63;
+#ifdef LVAR_ALT_PRIO
+  {
+    const int slot = __builtin_amdgcn_s_getreg(63492) & 1;  // hardware wave slot parity
+    const int round = (blockIdx.x / 512) & 1;
+    if (slot ^ round) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
+  }
+#endif
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, r = lane & 31;
   const int q0 = qt * WGROWS;

@@ -54,6 +54,34 @@ struct MaskListParams {
   int rows, nQ, nK, target;
 };
 
+struct TopkListParams {
+  const float* scores;  // [rows, n] with row stride score_stride
+  int32_t* indices;     // [rows, >= k] with row stride out_stride
+  int32_t* counts;      // [rows] or null
+  int64_t score_stride, out_stride;
+  int rows, n, k;
+};
+
+struct RemapListParams {
+  const int32_t* src;    // [BH, Gs, src_stride]
+  const int64_t* local;  // [Gk, local_stride] or null
+  int32_t* out;          // [BH*Gk, out_stride]
+  int32_t* counts;       // [BH*Gk] or null
+  int64_t src_stride, local_stride, out_stride;
+  int rows, Gs, Gk, cnt, rep, L, Lk;
+};
+
+struct MaskCompactParams {
+  const uint8_t* mask;  // [rows, n] with row stride mask_stride
+  int32_t* indices;     // [rows, out_len] with row stride out_stride
+  int32_t* counts;      // [rows]
+  int64_t mask_stride, out_stride;
+  int rows, n, out_len, multiple_of, zero_tail;
+};
+
+int launch_topk_token_lists(const TopkListParams& p, hipStream_t s);
+int launch_remap_concat_lists(const RemapListParams& p, hipStream_t s);
+int launch_mask_to_lists(const MaskCompactParams& p, hipStream_t s);
 int launch_block_topk_lists(const MaskListParams& p, hipStream_t s);
 int launch_attn(const AttnParams& p, int head_dim, int mode, bool accum, bool lse_only, int nwaves, hipStream_t s);
 int launch_colsum(const ColsumParams& p, int head_dim, hipStream_t s);

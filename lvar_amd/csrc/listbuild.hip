@@ -1,0 +1,221 @@
+// Key-list build on the GPU for the token-list attention path: exact per-row top-k selection of the
+// column sums, the cross-scale query-group remap fused with the local-run append, and the
+// compaction of a boolean mask into index lists.  All three are HBM/L2-bound integer work: one pass
+// (or a few L2-resident passes) over the rows, ballot/prefix compaction, no sorting.
+#include "common.h"
+#include "launch.h"
+
+namespace lvar {
+
+// Order-preserving map float -> uint32 (larger float <=> larger key); -0.0 sorts below +0.0.
+__device__ __forceinline__ uint32_t sort_key(float x) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+}
+
+__device__ __forceinline__ int lanes_below(unsigned long long bal, int lane) {
+  return __builtin_popcountll(bal & ((1ull << lane) - 1ull));
+}
+
+// ---------------------------------------------------------------------------------------------
+// Exact top-k per row by radix select.  One 256-thread workgroup per row; wave w owns the w-th
+// contiguous quarter of the (padded) row and every thread keeps its KPT keys in registers (KPT = 0:
+// rows too long for that are re-read from L2 in every pass).
+//   3 histogram passes (11, 11 and 10 bits, most significant first; LDS atomics) narrow the k-th
+//   largest key down to its exact value T and the number `need` of keys equal to T that belong to
+//   the selection (ties go to the smaller column);
+//   a counting pass gives every wave its number of selected keys, the last pass writes the selected
+//   columns in ascending order (ballot compaction).
+// ---------------------------------------------------------------------------------------------
+constexpr int TOPK_BINS = 2048;
+
+template <int KPT>
+__global__ __launch_bounds__(256) void topk_token_lists_kernel(const TopkListParams p) {
+  __shared__ int hist[TOPK_BINS];
+  __shared__ int wsum[4];
+  __shared__ int sel[2];  // chosen bin, keys still wanted inside it
+  __shared__ int wgt[4], weq[4];
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* s = p.scores + (int64_t)row * p.score_stride;
+  int32_t* out = p.indices + (int64_t)row * p.out_stride;
+  const int n = p.n;
+  int want = min(max(p.k, 0), n);  // keys still to be found among those matching the prefix
+  if (tid == 0 && p.counts) p.counts[row] = want;
+  if (want == 0) return;
+
+  // chunk c of wave w covers columns (w * cpw + c) * 64 .. +63
+  const int cpw = KPT ? KPT : ((n + 255) >> 8);
+  const int col0 = wave * cpw * 64 + lane;
+  uint32_t keys[KPT ? KPT : 1];
+  if (KPT) {
+#pragma unroll
+    for (int c = 0; c < KPT; c++) {
+      const int j = col0 + c * 64;
+      keys[c] = (j < n) ? sort_key(s[j]) : 0u;
+    }
+  }
+  // visit(f): f(chunk, column, key) for every chunk of this wave (all 64 lanes call it together)
+  auto visit = [&](auto&& f) {
+    if (KPT) {
+#pragma unroll
+      for (int c = 0; c < KPT; c++) f(col0 + c * 64, keys[c]);
+    } else {
+      for (int c = 0; c < cpw; c++) {
+        const int j = col0 + c * 64;
+        f(j, (j < n) ? sort_key(s[j]) : 0u);
+      }
+    }
+  };
+
+  uint32_t prefix = 0, pmask = 0;
+#pragma unroll
+  for (int pass = 0; pass < 3; pass++) {
+    const int shift = (pass == 0) ? 21 : (pass == 1) ? 10 : 0;
+    const int bits = (pass == 2) ? 10 : 11;
+    const int nbins = 1 << bits;
+    for (int t = tid; t < nbins; t += 256) hist[t] = 0;
+    __syncthreads();
+    visit([&](int j, uint32_t key) {
+      if (j < n && (key & pmask) == prefix) atomicAdd(&hist[(key >> shift) & (nbins - 1)], 1);
+    });
+    __syncthreads();
+    // thread t owns the bpt bins nbins-1 - t*bpt .. (descending); find the bin holding the want-th key from the top
+    const int bpt = nbins >> 8;
+    const int btop = nbins - 1 - tid * bpt;
+    int mine = 0;
+    for (int e = 0; e < bpt; e++) mine += hist[btop - e];
+    int incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int o = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += o;
+    }
+    if (lane == 63) wsum[wave] = incl;
+    __syncthreads();
+    int before = incl - mine;
+    for (int w = 0; w < wave; w++) before += wsum[w];
+    if (before < want && want <= before + mine) {  // exactly one thread
+      int acc = before, bin = btop;
+      for (int e = 0; e < bpt; e++) {
+        const int h = hist[btop - e];
+        if (acc + h >= want) { bin = btop - e; break; }
+        acc += h;
+      }
+      sel[0] = bin;
+      sel[1] = want - acc;
+    }
+    __syncthreads();
+    prefix |= (uint32_t)sel[0] << shift;
+    pmask |= (uint32_t)(nbins - 1) << shift;
+    want = sel[1];
+    __syncthreads();
+  }
+  const uint32_t T = prefix;  // key of the k-th largest element
+  const int need = want;      // selected keys equal to T (the first `need` of them by column)
+
+  int gt = 0, eq = 0;
+  visit([&](int j, uint32_t key) {
+    gt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(j < n && key > T));
+    eq += __builtin_popcountll(__builtin_amdgcn_ballot_w64(j < n && key == T));
+  });
+  if (lane == 0) { wgt[wave] = gt; weq[wave] = eq; }
+  __syncthreads();
+  int pos = 0, eq_before = 0;
+  for (int w = 0; w < wave; w++) {
+    pos += wgt[w] + max(0, min(weq[w], need - eq_before));
+    eq_before += weq[w];
+  }
+  int eq_left = max(0, need - eq_before);
+  visit([&](int j, uint32_t key) {
+    const bool is_gt = j < n && key > T, is_eq = j < n && key == T;
+    const unsigned long long beq = __builtin_amdgcn_ballot_w64(is_eq);
+    const bool keep = is_gt || (is_eq && lanes_below(beq, lane) < eq_left);
+    const unsigned long long bk = __builtin_amdgcn_ballot_w64(keep);
+    if (keep) out[pos + lanes_below(bk, lane)] = j;
+    pos += __builtin_popcountll(bk);
+    eq_left = max(0, eq_left - __builtin_popcountll(beq));
+  });
+}
+
+int launch_topk_token_lists(const TopkListParams& p, hipStream_t stream) {
+  if (p.rows == 0) return LVAR_OK;
+  const dim3 grid(p.rows), block(256);
+  if (p.n <= 256 * 8) hipLaunchKernelGGL(topk_token_lists_kernel<8>, grid, block, 0, stream, p);
+  else if (p.n <= 256 * 16) hipLaunchKernelGGL(topk_token_lists_kernel<16>, grid, block, 0, stream, p);
+  else if (p.n <= 256 * 32) hipLaunchKernelGGL(topk_token_lists_kernel<32>, grid, block, 0, stream, p);
+  else if (p.n <= 256 * 48) hipLaunchKernelGGL(topk_token_lists_kernel<48>, grid, block, 0, stream, p);
+  else if (p.n <= 256 * 64) hipLaunchKernelGGL(topk_token_lists_kernel<64>, grid, block, 0, stream, p);
+  else hipLaunchKernelGGL(topk_token_lists_kernel<0>, grid, block, 0, stream, p);
+  return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Sparse-step list: out[b,h,g, 0:cnt]       = clamp(src[b,h,gS(g), j / rep], 0, Lk-1)
+//                   out[b,h,g, cnt:cnt+L]   = local[g, 0:L]
+//                   counts[b,h,g]           = cnt + L
+// with gS(g) = clamp(rint((g + 0.5) / Gk * Gs - 0.5), 0, Gs-1) in fp32 (round half to even).
+// One workgroup per output row.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void remap_concat_lists_kernel(const RemapListParams p) {
+  const int row = blockIdx.x;  // bh * Gk + g
+  const int g = row % p.Gk, bh = row / p.Gk;
+  // three separately rounded fp32 operations (no fused multiply-add), as an eager tensor expression does
+  const float pos = __fsub_rn(__fmul_rn(__fdiv_rn((float)g + 0.5f, (float)p.Gk), (float)p.Gs), 0.5f);
+  const int gs = max(0, min(p.Gs - 1, (int)__builtin_rintf(pos)));
+  const int32_t* src = p.src + ((int64_t)bh * p.Gs + gs) * p.src_stride;
+  int32_t* out = p.out + (int64_t)row * p.out_stride;
+  for (int j = threadIdx.x; j < p.cnt; j += 256) out[j] = max(0, min(p.Lk - 1, src[j / p.rep]));
+  if (p.local) {
+    const int64_t* loc = p.local + (int64_t)g * p.local_stride;
+    for (int j = threadIdx.x; j < p.L; j += 256) out[p.cnt + j] = (int32_t)loc[j];
+  }
+  if (threadIdx.x == 0 && p.counts) p.counts[row] = p.cnt + (p.local ? p.L : 0);
+}
+
+int launch_remap_concat_lists(const RemapListParams& p, hipStream_t stream) {
+  if (p.rows == 0) return LVAR_OK;
+  hipLaunchKernelGGL(remap_concat_lists_kernel, dim3(p.rows), dim3(256), 0, stream, p);
+  return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Mask compaction: ascending columns of the set entries of a uint8 row, count rounded up to a
+// multiple with the lowest unset columns as padding.  One wave per row.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void mask_to_lists_kernel(const MaskCompactParams p) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  const uint8_t* m = p.mask + (int64_t)row * p.mask_stride;
+  int32_t* out = p.indices + (int64_t)row * p.out_stride;
+  const int chunks = (p.n + 63) >> 6;
+  int total = 0;
+  for (int c = 0; c < chunks; c++) {
+    const int j = c * 64 + lane;
+    const bool on = j < p.n && m[j] != 0;
+    const unsigned long long bal = __builtin_amdgcn_ballot_w64(on);
+    if (on) out[total + lanes_below(bal, lane)] = j;
+    total += __builtin_popcountll(bal);
+  }
+  const int mult = max(1, p.multiple_of);
+  const int padded = min(p.n, (total + mult - 1) / mult * mult);
+  int filled = total;
+  for (int c = 0; c < chunks && filled < padded; c++) {
+    const int j = c * 64 + lane;
+    const bool off = j < p.n && m[j] == 0;
+    const unsigned long long bal = __builtin_amdgcn_ballot_w64(off);
+    const int at = filled + lanes_below(bal, lane);
+    if (off && at < padded) out[at] = j;
+    filled = min(padded, filled + __builtin_popcountll(bal));
+  }
+  if (p.zero_tail)
+    for (int t = padded + lane; t < p.out_len; t += 64) out[t] = 0;
+  if (lane == 0) p.counts[row] = padded;
+}
+
+int launch_mask_to_lists(const MaskCompactParams& p, hipStream_t stream) {
+  if (p.rows == 0) return LVAR_OK;
+  hipLaunchKernelGGL(mask_to_lists_kernel, dim3(p.rows), dim3(64), 0, stream, p);
+  return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
+}
+
+}  // namespace lvar

@@ -41,20 +41,29 @@ def indices_count(top_keys: float, k_len: int, multiple_of: Optional[int] = None
 
 
 def topk_index_list(bs: torch.Tensor, top_keys: float, multiple_of: Optional[int] = None,
-                    indices_pad_to: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Full-step list build (models/sparvar/sparse_attn.py:1012-1036): descending top-k of the
-    colsum ``bs`` [B,H,G,Lk] -> ``inds`` int32 [B,H,G,Lk] whose first ``count`` columns are valid,
-    and ``counts`` int32 [B,H,G].  Padding columns are zero-filled (the reference leaves them
-    uninitialised; they are never read)."""
+                    indices_pad_to: Optional[int] = None, order: str = "value") -> Tuple[torch.Tensor, torch.Tensor]:
+    """Full-step list build (models/sparvar/sparse_attn.py:1012-1036): top-k of the colsum ``bs``
+    [B,H,G,Lk] -> ``inds`` int32 [B,H,G,Lk] whose first ``count`` columns are valid, and ``counts``
+    int32 [B,H,G].  Padding columns are zero-filled (the reference leaves them uninitialised; they
+    are never read).  ``order="value"`` lists the keys by descending score as ``torch.topk`` does,
+    ``order="index"`` by ascending key (same set; the attention kernels do not depend on the order
+    and gather ascending lists faster).  A tensor on a HIP device goes through the radix-select
+    kernel (:func:`lvar_amd.sparse_attn_ops.topk_token_lists`, ties to the smaller key)."""
     cfg = get_kernel_config_attn()
     m = cfg["counts_multiple_of"] if multiple_of is None else multiple_of
     B, H, G, Lk = bs.shape
     cnt = indices_count(top_keys, Lk, m)
     if cnt > Lk:
         raise ValueError(f"top-k count {cnt} exceeds key length {Lk}")
+    if order not in ("value", "index"):
+        raise ValueError("order must be 'value' or 'index'")
+    if bs.is_cuda:
+        from . import sparse_attn_ops as ops
+        return ops.topk_token_lists(bs, cnt, out_len=Lk, order=order)
     inds = torch.zeros((B, H, G, Lk), dtype=torch.int32, device=bs.device)
     if cnt > 0:
-        inds[..., :cnt] = torch.topk(bs, k=cnt, dim=-1).indices.to(torch.int32)
+        top = torch.topk(bs, k=cnt, dim=-1).indices
+        inds[..., :cnt] = (top if order == "value" else top.sort(-1).values).to(torch.int32)
     counts = torch.full((B, H, G), cnt, dtype=torch.int32, device=bs.device)
     return inds, counts
 
@@ -184,7 +193,11 @@ def flex_block_mask(q_scale_idx: int, kernel_schedule: Sequence[int], attn_sink_
 
 def block_mask_to_lists(mask: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """bool [..., nQ, nK] -> flex ``BlockMask`` lists: ``kv_num_blocks`` int32 [..., nQ] and
-    ``kv_indices`` int32 [..., nQ, nK] (kept blocks first, ascending; unused tail zero)."""
+    ``kv_indices`` int32 [..., nQ, nK] (kept blocks first, ascending; unused tail zero).  A mask on
+    a HIP device is compacted by one kernel (:func:`lvar_amd.sparse_attn_ops.mask_to_lists`)."""
+    if mask.is_cuda:
+        from . import sparse_attn_ops as ops
+        return ops.mask_to_lists(mask, 1)
     nK = mask.shape[-1]
     num = mask.sum(-1, dtype=torch.int32)
     # kept blocks sort before dropped ones, both in ascending block order

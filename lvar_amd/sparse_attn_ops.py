@@ -272,3 +272,90 @@ def block_topk_lists(block_scores, target: int, base_mask=None):
                                               B, H, nQ, nK, int(target), _stream(bs))
     _lib.check(st, "lvar_block_topk_lists")
     return num, idx
+
+
+def topk_token_lists(scores, k: int, out_len: Optional[int] = None, order: str = "index"):
+    """Exact top-``k`` key columns of every row of ``scores`` (fp32 ``[..., Lk]``, e.g. the column sums
+    ``[B,H,G,Lk]``) on the GPU: returns ``(indices int32 [..., out_len], counts int32 [...])`` with the
+    selected columns in the first ``k`` entries (``out_len`` defaults to ``Lk``, the width the list
+    attention op expects; entries beyond ``k`` are zero).  ``order="index"`` (default, one kernel)
+    lists them in ascending column order, which is also the best order for the gather kernel;
+    ``order="value"`` re-orders them by descending score like ``torch.topk``
+    (models/sparvar/sparse_attn.py:1016).  Ties at the k-th value go to the smaller column."""
+    _require(scores.dim() >= 1, "scores must have a key axis")
+    if not scores.is_cuda:
+        raise RuntimeError("scores must live on a HIP device; lvar_amd has no CPU path")
+    _require(order in ("index", "value"), "order must be 'index' or 'value'")
+    sc = scores.to(torch.float32).contiguous()
+    Lk = sc.shape[-1]
+    rows = sc.numel() // Lk if Lk else 0
+    k = int(k)
+    _require(0 <= k <= Lk, f"k = {k} must lie in [0, Lk = {Lk}]")
+    out_len = Lk if out_len is None else int(out_len)
+    _require(out_len >= k, "out_len must be at least k")
+    idx = torch.zeros(sc.shape[:-1] + (out_len,), dtype=torch.int32, device=sc.device)
+    cnt = torch.empty(sc.shape[:-1], dtype=torch.int32, device=sc.device)
+    with torch.cuda.device(sc.device):
+        st = _lib.load().lvar_topk_token_lists(sc.data_ptr(), Lk, idx.data_ptr(), out_len, cnt.data_ptr(),
+                                              rows, Lk, k, _stream(sc))
+    _lib.check(st, "lvar_topk_token_lists")
+    if order == "value" and k > 0:
+        sel = idx[..., :k].long()
+        vals = sc.gather(-1, sel)
+        perm = torch.sort(vals, dim=-1, descending=True, stable=True).indices
+        idx[..., :k] = sel.gather(-1, perm).to(torch.int32)
+    return idx, cnt
+
+
+def remap_concat_lists(src_indices, src_count: int, cur_q_len: int, cur_k_len: int, local_indices=None,
+                       bm: int = 192, indices_pad_to: int = 1, out_len: Optional[int] = None):
+    """One-launch sparse-step key list: the decision-scale lists ``src_indices`` int32 ``[B,H,Gs,Ks]``
+    (first ``src_count`` columns valid) are mapped to the ``Gk = ceil(cur_q_len / bm)`` query groups of the
+    current scale (nearest group centre, half-to-even), clamped to ``[0, cur_k_len)``, and followed by
+    the rows of ``local_indices`` int64 ``[Gk, L]`` (optional).  Returns ``(indices int32 [B,H,Gk,out_len],
+    counts int32 [B,H,Gk])``; ``out_len`` defaults to ``cur_k_len``.  Equals
+    ``append_local_run(map_inds_counts_across_scales(...))`` of :mod:`lvar_amd.mask_build`
+    (models/sparvar/sparse_attn.py:366-421, 1096-1121)."""
+    _require(src_indices.dim() == 4, "src_indices must be [B,H,Gs,Ks]")
+    if not src_indices.is_cuda:
+        raise RuntimeError("src_indices must live on a HIP device; lvar_amd has no CPU path")
+    src = src_indices.to(torch.int32).contiguous()
+    B, H, Gs, Ks = src.shape
+    Gk = (int(cur_q_len) + bm - 1) // bm
+    raw = int(src_count)
+    cnt = max(indices_pad_to, (raw + indices_pad_to - 1) // indices_pad_to * indices_pad_to)
+    L = 0
+    loc = None
+    if local_indices is not None:
+        _require(local_indices.dim() == 2 and local_indices.shape[0] == Gk, f"local_indices must be [Gk = {Gk}, L]")
+        loc = local_indices.to(device=src.device, dtype=torch.int64).contiguous()
+        L = loc.shape[1]
+    out_len = int(cur_k_len) if out_len is None else int(out_len)
+    _require(cnt + L <= out_len, f"list length {cnt + L} exceeds the output width {out_len}")
+    out = torch.zeros((B, H, Gk, out_len), dtype=torch.int32, device=src.device)
+    counts = torch.empty((B, H, Gk), dtype=torch.int32, device=src.device)
+    with torch.cuda.device(src.device):
+        st = _lib.load().lvar_remap_concat_lists(src.data_ptr(), Ks, Ks, _ptr(loc), L, L, out.data_ptr(), out_len,
+                                                counts.data_ptr(), B * H, Gs, Gk, cnt, int(cur_k_len), _stream(src))
+    _lib.check(st, "lvar_remap_concat_lists")
+    return out, counts
+
+
+def mask_to_lists(mask, multiple_of: int = 1):
+    """Compaction of a boolean mask ``[..., n]`` on the GPU: ``(counts int32 [...], indices int32 [..., n])``
+    with the ascending set columns first, the count rounded up to ``multiple_of`` with the lowest unset
+    columns as padding, and a zero tail.  For a block mask ``[B,H,nQ,nK]`` and ``multiple_of = 1`` these are
+    the flex ``BlockMask`` lists ``(kv_num_blocks, kv_indices)`` taken by :func:`block_sparse_attn`
+    (kernels/chipmunk/csrc/indexed_io/mask_to_indices.cu:21-97)."""
+    if not mask.is_cuda:
+        raise RuntimeError("mask must live on a HIP device; lvar_amd has no CPU path")
+    m = mask.to(torch.uint8).contiguous()
+    n = m.shape[-1]
+    rows = m.numel() // n if n else 0
+    idx = torch.empty(m.shape, dtype=torch.int32, device=m.device)
+    cnt = torch.empty(m.shape[:-1], dtype=torch.int32, device=m.device)
+    with torch.cuda.device(m.device):
+        st = _lib.load().lvar_mask_to_lists(m.data_ptr(), n, idx.data_ptr(), n, cnt.data_ptr(), rows, n,
+                                           int(multiple_of), _stream(m))
+    _lib.check(st, "lvar_mask_to_lists")
+    return cnt, idx

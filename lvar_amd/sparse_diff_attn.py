@@ -34,6 +34,7 @@ class SparseDiffAttn:
         self.dense_colsum_attn = ops.dense_colsum_attn_s if speedup else ops.dense_colsum_attn_q
         self.indices = None
         self.counts = None
+        self.count_host = 0
         self.out_cache = None
 
     def forward(self, q, k, v, scale, do_full_step: bool = False, inference_step: int = 0, scale_ind: int = 0, layer_ind: int = 0):
@@ -42,24 +43,31 @@ class SparseDiffAttn:
         top_keys = GLOBAL_CONFIG["attn"]["top_keys"]
         if do_full_step:                                           # sparse_attn.py:991-1051
             o, bs = self.dense_colsum_attn(q, k, v, scale)
-            inds, counts = mb.topk_index_list(bs, top_keys, self.multiple_of, self.indices_pad_to)
+            inds, counts = mb.topk_index_list(bs, top_keys, self.multiple_of, self.indices_pad_to, order="index")
             self.indices, self.counts = inds, counts
+            self.count_host = mb.indices_count(top_keys, k.shape[-2], self.multiple_of)
             if self.use_o_cache:
                 # O_cache = O_dense + (-1) * delta(O) over the selected keys
                 self.out_cache = ops.csp_attn(q, k, v, scale, inds, counts, o, -1)
             return o
         # sparse step, sparse_attn.py:1053-1144
         inds, counts = self.indices, self.counts
-        s_count = int(counts[0, 0, 0])
+        s_count = self.count_host                                  # the reference reads counts[0,0,0] back (a host sync)
         if inds.shape[0] != q.shape[0]:
             inds, counts = inds[:q.shape[0]], counts[:q.shape[0]]
-        inds, counts = mb.map_inds_counts_across_scales(inds, s_count, cur_q_len=q.shape[-2], cur_k_len=k.shape[-2],
-                                                        bm=self.bm, indices_pad_to=self.indices_pad_to)
         local_inds, local_count = self.local_inds[scale_ind]
-        inds, counts = mb.append_local_run(inds, inds.shape[-1], local_inds, local_count,
-                                           k_len=k.shape[-2], multiple_of=self.multiple_of)
+        if local_inds.device != inds.device:
+            local_inds = local_inds.to(inds.device)
+            self.local_inds[scale_ind] = (local_inds, local_count)
+        # group remap + clamp + local-run append + counts in one launch (sparse_attn.py:1056-1121)
+        inds, counts = ops.remap_concat_lists(inds, s_count, q.shape[-2], k.shape[-2], local_inds,
+                                              bm=self.bm, indices_pad_to=self.indices_pad_to)
+        assert int(inds.shape[-1]) >= s_count + local_count and (s_count + local_count) % self.multiple_of == 0, \
+            f"after add local sparse index, mismatch multiple_of={self.multiple_of}"
         if scale_ind != len(self.scales) - 1:
             self.indices, self.counts = inds, counts               # cached for the next scale
+            pad = self.indices_pad_to
+            self.count_host = max(pad, (s_count + pad - 1) // pad * pad) + local_count
         if self.use_o_cache:
             o = self.out_cache
             if o.shape[0] != q.shape[0]:

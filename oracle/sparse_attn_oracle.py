@@ -28,6 +28,7 @@ __all__ = [
     "map_inds_counts_across_scales", "local_window_indices", "crossscale_self_indices",
     "aggregate_group_indices", "upsample_ocache", "flex_block_mask", "infinity_cum",
     "INFINITY_SCALES", "config2_block_mask", "attn_flops_blocks", "attn_flops_lists",
+    "topk_token_set", "append_local_run", "mask_to_lists",
 ]
 
 # Infinity "1M" scale schedule, reference utils/dynamic_resolution.py:7 and
@@ -260,6 +261,53 @@ def map_inds_counts_across_scales(inds_S, counts_S, cur_q_len, cur_k_len, bm=192
     out.clamp_(0, max(0, cur_k_len - 1))
     counts = torch.full((B, H, Gk), cnt, dtype=torch.int32)
     return out, counts
+
+
+def topk_token_set(scores, k):
+    """Columns of the k largest entries of each row, ascending: the SET ``torch.topk(bs, k)`` selects
+    in the full step (models/sparvar/sparse_attn.py:1016), with the one freedom torch leaves open
+    (ties at the k-th value) fixed to "smaller column first", i.e. the first k entries of a stable
+    descending sort.  ``scores`` [..., n] -> int32 [..., k]."""
+    x = np.asarray(scores.detach().to(torch.float32).cpu().numpy())
+    flat = x.reshape(-1, x.shape[-1])
+    out = np.zeros((flat.shape[0], k), dtype=np.int32)
+    for r in range(flat.shape[0]):
+        order = np.argsort(-flat[r], kind="stable")      # descending by value, equal values by column
+        out[r] = np.sort(order[:k])
+    return torch.from_numpy(out.reshape(x.shape[:-1] + (k,)))
+
+
+def append_local_run(inds, count, local_inds, local_count, k_len):
+    """Sparse-step list: the first ``count`` remapped top-k keys followed by the scale's local run, zero
+    padded to ``k_len`` columns (models/sparvar/sparse_attn.py:1096-1121).  inds [B,H,G,>=count],
+    local_inds [G, local_count] -> (int32 [B,H,G,k_len], counts int32 [B,H,G])."""
+    B, H, G, _ = inds.shape
+    out = torch.zeros(B, H, G, k_len, dtype=torch.int32)
+    for g in range(G):
+        out[:, :, g, :count] = inds[:, :, g, :count].to(torch.int32)
+        out[:, :, g, count:count + local_count] = local_inds[g, :local_count].to(torch.int32)
+    return out, torch.full((B, H, G), count + local_count, dtype=torch.int32)
+
+
+def mask_to_lists(mask, multiple_of=1):
+    """Row-wise mask compaction with count padding, as the reference's mask_to_indices kernel
+    (kernels/chipmunk/csrc/indexed_io/mask_to_indices.cu:21-97): ascending set columns, then the lowest
+    unset columns until the count is a multiple of ``multiple_of`` (capped at the row length); the
+    rest of the row is zero here (the reference leaves it untouched).  Pure-Python loops.
+    bool [..., n] -> (counts int32 [...], indices int32 [..., n])."""
+    m = np.asarray(mask.detach().cpu().numpy()).astype(bool)
+    n = m.shape[-1]
+    flat = m.reshape(-1, n)
+    idx = np.zeros((flat.shape[0], n), dtype=np.int32)
+    cnt = np.zeros((flat.shape[0],), dtype=np.int32)
+    for r in range(flat.shape[0]):
+        on = [j for j in range(n) if flat[r, j]]
+        off = [j for j in range(n) if not flat[r, j]]
+        padded = min(n, (len(on) + multiple_of - 1) // multiple_of * multiple_of)
+        row = on + off[:padded - len(on)]
+        idx[r, :len(row)] = row
+        cnt[r] = len(row)
+    return torch.from_numpy(cnt.reshape(m.shape[:-1])), torch.from_numpy(idx.reshape(m.shape))
 
 
 def local_window_indices(Hh, W, base, win):

@@ -102,3 +102,64 @@ def test_torch_ops_chipmunk_schemas():
     assert close(oc, ref) and not torch.equal(oc, o)
     with pytest.raises(Exception):
         torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds.cuda(), counts.cuda(), 2)
+
+
+@pytest.mark.gpu
+def test_topk_token_lists_matches_oracle_set():
+    """GPU radix select against the oracle's stable-sort selection: bit-exact index lists, with
+    ties through the cut, k = 0, k = Lk, a ragged Lk, and the descending-by-value order option."""
+    import oracle
+    from lvar_amd import sparse_attn_ops as ops
+    g = torch.Generator().manual_seed(5)
+    for (shape, k) in (((2, 3, 4, 1000), 192), ((1, 2, 22, 10521), 2112), ((3, 777), 0), ((3, 777), 777), ((5, 130), 1),
+                       ((2, 20000), 4000), ((2, 41000), 513)):   # > 48 KB of LDS; beyond the LDS-staged limit
+        x = torch.rand(*shape, generator=g)
+        if shape[-1] == 1000:
+            x[0, 0, 0] = torch.tensor([1.0, 2.0] * 500)                   # half the row tied at the cut
+            x[1, 2, 3] = 0.5                                              # constant row
+            x[0, 1, 1, ::3] = -x[0, 1, 1, ::3]                            # negative values
+        idx, cnt = ops.topk_token_lists(x.cuda(), k)
+        assert idx.shape == shape and cnt.shape == shape[:-1] and bool((cnt == k).all())
+        exp = oracle.topk_token_set(x, k)
+        assert torch.equal(idx[..., :k].cpu(), exp), (shape, k)
+        assert bool((idx[..., k:] == 0).all())
+    x = torch.rand(2, 2, 3, 500, generator=g)
+    idx, _ = ops.topk_token_lists(x.cuda(), 64, order="value")
+    assert torch.equal(idx[..., :64].cpu().long(), torch.topk(x, 64, dim=-1).indices)   # distinct values: same order
+    with pytest.raises(AssertionError):
+        ops.topk_token_lists(x.cuda(), 501)
+
+
+@pytest.mark.gpu
+def test_remap_concat_lists_matches_oracle():
+    import oracle
+    from lvar_amd import sparse_attn_ops as ops
+    g = torch.Generator().manual_seed(6)
+    # decision scale 40x40 (Lq 1600, Gs 9) -> scales 48 (Gk 12) and 64 (Gk 22); Ks >= count and Ks < count
+    for (Gs, Ks, count, q_len, k_len, L, pad) in ((9, 4121, 832, 2304, 6425, 448, 1), (9, 4121, 832, 4096, 10521, 672, 1),
+                                                  (9, 100, 250, 4096, 10521, 0, 4), (1, 64, 64, 192, 300, 64, 1)):
+        src = torch.randint(0, k_len + 50, (2, 3, Gs, Ks), generator=g, dtype=torch.int32)   # some beyond Lk: clamped
+        Gk = (q_len + 191) // 192
+        local = torch.randint(0, k_len, (Gk, L), generator=g) if L else None
+        counts_S = torch.full((2, 3, Gs), count, dtype=torch.int32)
+        e_idx, e_cnt = oracle.map_inds_counts_across_scales(src, counts_S, q_len, k_len, 192, pad)
+        cnt = int(e_cnt[0, 0, 0])
+        if L:
+            e_idx, e_cnt = oracle.append_local_run(e_idx, cnt, local, L, k_len)
+        out, counts = ops.remap_concat_lists(src.cuda(), count, q_len, k_len, local.cuda() if L else None, 192, pad)
+        assert out.shape == (2, 3, Gk, k_len)
+        assert torch.equal(counts.cpu(), e_cnt)
+        assert torch.equal(out[..., :cnt + L].cpu(), e_idx[..., :cnt + L])
+        assert bool((out[..., cnt + L:] == 0).all())
+
+
+@pytest.mark.gpu
+def test_mask_to_lists_matches_oracle():
+    import oracle
+    from lvar_amd import sparse_attn_ops as ops
+    g = torch.Generator().manual_seed(7)
+    for shape, p, mult in (((2, 2, 32, 165), 0.25, 1), ((3, 5, 700), 0.2, 64), ((4, 64), 0.0, 8), ((4, 65), 1.0, 8), ((2, 130), 0.97, 112)):
+        m = torch.rand(*shape, generator=g) < p
+        cnt, idx = ops.mask_to_lists(m.cuda(), mult)
+        e_cnt, e_idx = oracle.mask_to_lists(m, mult)
+        assert torch.equal(cnt.cpu(), e_cnt) and torch.equal(idx.cpu(), e_idx), (shape, p, mult)

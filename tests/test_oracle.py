@@ -247,3 +247,50 @@ def test_config2_block_mask_density():
             rest = scores[0, h, i].masked_fill(base[0, h, i], -1.0)
             best = torch.sort(rest, descending=True).indices[:extra.numel()]
             assert sorted(extra.tolist()) == sorted(best.tolist())
+
+
+def test_topk_token_set_against_rank_definition_and_torch_topk():
+    """The selected set is pinned by the rank definition (brute force) and, where all values are
+    distinct, by torch.topk (library); ties go to the smaller column."""
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(3, 2, 57, generator=g)
+    x[0, 0, 5] = x[0, 0, 40] = x[0, 0, 41] = x[0, 0].max() + 1.0       # ties above the cut
+    x[1, 1, :] = torch.tensor([1.0, 2.0] * 28 + [1.0])                   # heavy ties through the cut
+    for k in (0, 1, 7, 29, 57):
+        got = oracle.topk_token_set(x, k)
+        assert got.shape == (3, 2, k) and got.dtype == torch.int32
+        for r in range(3):
+            for c in range(2):
+                row = x[r, c].tolist()
+                exp = [j for j in range(57)
+                       if sum(1 for t in range(57) if row[t] > row[j] or (row[t] == row[j] and t < j)) < k]
+                assert got[r, c].tolist() == exp
+        if k:
+            ref = torch.topk(x[2], k, dim=-1).indices.sort(-1).values      # rows of x[2] have distinct values
+            assert torch.equal(got[2].long(), ref)
+
+
+def test_mask_to_lists_small_cases():
+    m = torch.tensor([[0, 1, 0, 1, 1, 0, 0, 0], [0, 0, 0, 0, 0, 0, 0, 0], [1, 1, 1, 1, 1, 1, 1, 1]], dtype=torch.bool)
+    cnt, idx = oracle.mask_to_lists(m, 1)
+    assert cnt.tolist() == [3, 0, 8]
+    assert idx.tolist() == [[1, 3, 4, 0, 0, 0, 0, 0], [0] * 8, list(range(8))]
+    cnt, idx = oracle.mask_to_lists(m, 4)                                # pad with the lowest unset columns
+    assert cnt.tolist() == [4, 0, 8]
+    assert idx[0].tolist() == [1, 3, 4, 0, 0, 0, 0, 0]
+    cnt, idx = oracle.mask_to_lists(m, 5)
+    assert cnt.tolist() == [5, 0, 8] and idx[0].tolist() == [1, 3, 4, 0, 2, 0, 0, 0]
+    # multiple_of = 1 on a block mask equals the flex BlockMask lists of block_mask_to_lists
+    g = torch.Generator().manual_seed(3)
+    bm = torch.rand(2, 3, 5, 19, generator=g) < 0.3
+    num, bidx = oracle.block_mask_to_lists(bm)
+    cnt, idx = oracle.mask_to_lists(bm, 1)
+    assert torch.equal(cnt, num) and torch.equal(idx, bidx)
+
+
+def test_append_local_run_layout():
+    inds = torch.arange(2 * 1 * 3 * 10, dtype=torch.int32).reshape(2, 1, 3, 10)
+    local = torch.tensor([[100, 101], [200, 201], [300, 301]])
+    out, counts = oracle.append_local_run(inds, 4, local, 2, 9)
+    assert out.shape == (2, 1, 3, 9) and counts.tolist() == [[[6] * 3]] * 2
+    assert out[1, 0, 2].tolist() == [50, 51, 52, 53, 300, 301, 0, 0, 0]
