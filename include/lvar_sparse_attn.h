@@ -89,6 +89,26 @@ int lvar_csp_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v,
                       float o_scale, float scale, void* stream);
 
 /*
+ * Token-list attention of a sparse step with the O-cache resampled in the epilogue:
+ *   o[b,h,i,:] = bilinear(o_cache[b,h])(y_i, x_i) + o_scale * softmax(q_i k[idx]^T scale) v[idx],
+ * where o_cache [B,H,src_side*src_side,head_dim] (bf16) is the cached attention output of a coarser
+ * src_side x src_side token grid, the Lq = dst_side*dst_side queries form a dst_side x dst_side grid
+ * (i = y_i*dst_side + x_i), and the resampling uses half-pixel centres with edge clamp
+ * (source coordinate max(0, (t+0.5)*src_side/dst_side - 0.5): torch's bilinear, align_corners=False).
+ * The four taps are read in the attention epilogue and combined in fp32, so the upsampled cache
+ * is never written to memory and o is rounded once.  Other arguments as lvar_csp_attn_fwd.
+ * Replaces upsample_Ocache(...).to(v.dtype) followed by csp_attn(q,k,v,scale,inds,counts,o,1)
+ * (models/sparvar/sparse_attn.py:324-362, 1129-1142).
+ */
+int lvar_csp_attn_upsample_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v,
+                               lvar_tensor_t o_cache, int src_side, int dst_side,
+                               lvar_tensor_t o, float* M, float* L,
+                               const int32_t* indices, const int32_t* counts,
+                               int G, int64_t idx_row_stride, int group_rows,
+                               int B, int H, int Lq, int Lk, int head_dim,
+                               float o_scale, float scale, void* stream);
+
+/*
  * Block-sparse attention over a compacted per-query-block list of key blocks in the flex
  * BlockMask layout consumed by SparseFlexAttn (models/sparvar/basic_sparvar.py:55-72,187-194):
  * kv_num_blocks int32 [B,H,nQ] (stride_nb_b, stride_nb_h, 1), kv_indices int32

@@ -12,7 +12,8 @@ from .build import LIB_PATH
 
 EXPORTED_SYMBOLS = (
     "lvar_version", "lvar_target_arch", "lvar_status_string",
-    "lvar_dense_attn_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_block_sparse_attn_fwd",
+    "lvar_dense_attn_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_csp_attn_upsample_fwd",
+    "lvar_block_sparse_attn_fwd",
     "lvar_block_topk_lists", "lvar_topk_token_lists", "lvar_remap_concat_lists", "lvar_mask_to_lists",
 )
 
@@ -53,6 +54,8 @@ def load() -> C.CDLL:
     lib.lvar_colsum_fwd.argtypes = [T, T, P, P, P, I, I, I, I, I, I, F, P]
     lib.lvar_csp_attn_fwd.restype = I
     lib.lvar_csp_attn_fwd.argtypes = [T, T, T, T, T, P, P, P, P, I, I64, I, I, I, I, I, I, F, F, P]
+    lib.lvar_csp_attn_upsample_fwd.restype = I
+    lib.lvar_csp_attn_upsample_fwd.argtypes = [T, T, T, T, I, I, T, P, P, P, P, I, I64, I, I, I, I, I, I, F, F, P]
     lib.lvar_block_sparse_attn_fwd.restype = I
     lib.lvar_block_sparse_attn_fwd.argtypes = [T, T, T, T, P, P, P, I64, I64, P, I64, I64, I64, I, I, I, I, I, I, I, I, F, P]
     lib.lvar_block_topk_lists.restype = I

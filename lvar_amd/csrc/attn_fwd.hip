@@ -439,8 +439,29 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const float osc = ACCUM ? p.o_scale * inv : inv;
   char* ob = smem + wave * (32 * OSTR);
   const bf16_t* oap = nullptr;
-  if (ACCUM && p.o_accum)
-    oap = p.o_accum + b * p.oa_sb + h * p.oa_sh + (int64_t)min(qrow_w, p.Lq - 1) * p.oa_sr;
+  // bilinear taps of this lane's query in a coarser o_accum grid (half-pixel centres, edge clamp:
+  // src = max(0, (dst + 0.5) * src_side / dst_side - 0.5), the align_corners = False rule)
+  const bf16_t *tap01 = nullptr, *tap10 = nullptr, *tap11 = nullptr;
+  float wy1 = 0.f, wx1 = 0.f;
+  if (ACCUM && p.o_accum) {
+    const bf16_t* base = p.o_accum + b * p.oa_sb + h * p.oa_sh;
+    const int qr = min(qrow_w, p.Lq - 1);
+    if (p.up_src > 0) {
+      const int y = qr / p.up_dst, x = qr - y * p.up_dst;
+      const float sc = (float)p.up_src / (float)p.up_dst;
+      const float sy = fmaxf(sc * ((float)y + 0.5f) - 0.5f, 0.f), sx = fmaxf(sc * ((float)x + 0.5f) - 0.5f, 0.f);
+      const int y0 = min((int)sy, p.up_src - 1), x0 = min((int)sx, p.up_src - 1);
+      const int y1 = min(y0 + 1, p.up_src - 1), x1 = min(x0 + 1, p.up_src - 1);
+      wy1 = sy - (float)y0;
+      wx1 = sx - (float)x0;
+      oap = base + (int64_t)(y0 * p.up_src + x0) * p.oa_sr;
+      tap01 = base + (int64_t)(y0 * p.up_src + x1) * p.oa_sr;
+      tap10 = base + (int64_t)(y1 * p.up_src + x0) * p.oa_sr;
+      tap11 = base + (int64_t)(y1 * p.up_src + x1) * p.oa_sr;
+    } else {
+      oap = base + (int64_t)qr * p.oa_sr;
+    }
+  }
 #pragma unroll
   for (int m = 0; m < MTD; m++) {
 #pragma unroll
@@ -450,8 +471,16 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       float x2 = oacc[m][4 * a + 2] * osc, x3 = oacc[m][4 * a + 3] * osc;
       if (ACCUM && oap) {
         u32x2 acc = *(const u32x2*)(oap + dcol);
-        x0 += bf16_lo(acc[0]); x1 += bf16_hi(acc[0]);
-        x2 += bf16_lo(acc[1]); x3 += bf16_hi(acc[1]);
+        float a0 = bf16_lo(acc[0]), a1 = bf16_hi(acc[0]), a2 = bf16_lo(acc[1]), a3 = bf16_hi(acc[1]);
+        if (tap01) {
+          const u32x2 t01 = *(const u32x2*)(tap01 + dcol), t10 = *(const u32x2*)(tap10 + dcol), t11 = *(const u32x2*)(tap11 + dcol);
+          const float wy0 = 1.f - wy1, wx0 = 1.f - wx1;
+          a0 = wy0 * (wx0 * a0 + wx1 * bf16_lo(t01[0])) + wy1 * (wx0 * bf16_lo(t10[0]) + wx1 * bf16_lo(t11[0]));
+          a1 = wy0 * (wx0 * a1 + wx1 * bf16_hi(t01[0])) + wy1 * (wx0 * bf16_hi(t10[0]) + wx1 * bf16_hi(t11[0]));
+          a2 = wy0 * (wx0 * a2 + wx1 * bf16_lo(t01[1])) + wy1 * (wx0 * bf16_lo(t10[1]) + wx1 * bf16_lo(t11[1]));
+          a3 = wy0 * (wx0 * a3 + wx1 * bf16_hi(t01[1])) + wy1 * (wx0 * bf16_hi(t10[1]) + wx1 * bf16_hi(t11[1]));
+        }
+        x0 += a0; x1 += a1; x2 += a2; x3 += a3;
       }
       u32x2 pk = {pack_bf16(x0, x1), pack_bf16(x2, x3)};
       *(u32x2*)(ob + r * OSTR + dcol * 2) = pk;

@@ -92,8 +92,8 @@ int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* 
   return launch_colsum(p, head_dim, (hipStream_t)stream);
 }
 
-int lvar_csp_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o_accum, lvar_tensor_t o,
-                      float* M, float* L, const int32_t* indices, const int32_t* counts, int G,
+static int csp_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o_accum, int up_src, int up_dst,
+                      lvar_tensor_t o, float* M, float* L, const int32_t* indices, const int32_t* counts, int G,
                       int64_t idx_row_stride, int group_rows, int B, int H, int Lq, int Lk, int head_dim,
                       float o_scale, float scale, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
@@ -113,12 +113,33 @@ int lvar_csp_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_te
   p.cnt_sh = G; p.cnt_sb = (int64_t)H * G;
   p.list_len = (int)(idx_row_stride > 0x7fffffff ? 0x7fffffff : idx_row_stride);
   p.group_rows = group_rows;
+  p.up_src = up_src; p.up_dst = up_dst;
   int nw = gather_waves();
   while (group_rows % (nw * 32) != 0) nw = (nw == 6) ? 3 : (nw == 3 ? 2 : 1);
   if (nw == 1) {
     if (group_rows % 64 == 0) nw = 2; else return LVAR_EUNSUPPORTED;
   }
   return launch_attn(p, head_dim, MODE_GATHER, true, false, nw, (hipStream_t)stream);
+}
+
+int lvar_csp_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o_accum, lvar_tensor_t o,
+                      float* M, float* L, const int32_t* indices, const int32_t* counts, int G,
+                      int64_t idx_row_stride, int group_rows, int B, int H, int Lq, int Lk, int head_dim,
+                      float o_scale, float scale, void* stream) {
+  return csp_common(q, k, v, o_accum, 0, 0, o, M, L, indices, counts, G, idx_row_stride, group_rows, B, H, Lq, Lk,
+                    head_dim, o_scale, scale, stream);
+}
+
+int lvar_csp_attn_upsample_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o_cache,
+                               int src_side, int dst_side, lvar_tensor_t o, float* M, float* L,
+                               const int32_t* indices, const int32_t* counts, int G, int64_t idx_row_stride,
+                               int group_rows, int B, int H, int Lq, int Lk, int head_dim,
+                               float o_scale, float scale, void* stream) {
+  if (!o_cache.ptr || src_side <= 0 || dst_side <= 0 || src_side > 32768 || dst_side > 32768 ||
+      (int64_t)dst_side * dst_side != Lq)
+    return LVAR_EINVAL;
+  return csp_common(q, k, v, o_cache, src_side, dst_side, o, M, L, indices, counts, G, idx_row_stride, group_rows,
+                    B, H, Lq, Lk, head_dim, o_scale, scale, stream);
 }
 
 int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,

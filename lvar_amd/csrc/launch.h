@@ -30,6 +30,8 @@ struct AttnParams {
   int list_len;    // entries available per list row; counts are clamped to it
   int group_rows;  // query rows sharing one list
   int sub_shift;   // log2(64-key tiles per key block)
+  int up_src, up_dst;  // token-list variant: o_accum is an up_src x up_src token grid, bilinearly
+                       // resampled to the up_dst x up_dst grid of the queries (0 = o_accum has Lq rows)
   int nqt, total_wg;
 };
 

@@ -162,7 +162,7 @@ def dense_colsum_attn_q(q, k, v, scale=None):
     return dense_colsum_attn_s(q, k, v, scale)
 
 
-def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats):
+def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, upsample_from=None):
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
     _check_qkv(q, k, v)
     B, H, Lq, d = q.shape
@@ -182,17 +182,29 @@ def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats):
     counts = counts.contiguous()
     if o_accum is not None:
         o_accum = _prep(o_accum, "o")
-        _require(o_accum.shape == q.shape, f"Output shape mismatch - o: {tuple(o_accum.shape)}, q: {tuple(q.shape)}")
+        if upsample_from is None:
+            _require(o_accum.shape == q.shape, f"Output shape mismatch - o: {tuple(o_accum.shape)}, q: {tuple(q.shape)}")
+        else:
+            src, dst = upsample_from
+            _require(dst * dst == Lq and tuple(o_accum.shape) == (B, H, src * src, d),
+                     f"O-cache shape mismatch - o_cache: {tuple(o_accum.shape)}, expected {(B, H, src * src, d)} "
+                     f"for a {src}x{src} -> {dst}x{dst} grid, q: {tuple(q.shape)}")
     o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device)
     M = L = None
     if want_stats:
         M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
         L = torch.empty_like(M)
     with torch.cuda.device(q.device):
-        st = _lib.load().lvar_csp_attn_fwd(_view(q), _view(k), _view(v), _view(o_accum), _view(o), _ptr(M), _ptr(L),
-                                          indices.data_ptr(), counts.data_ptr(), G, indices.stride(2), bm,
-                                          B, H, Lq, Lk, d, float(o_scale), _scale(q, scale), _stream(q))
-    _lib.check(st, "lvar_csp_attn_fwd")
+        if upsample_from is None:
+            st = _lib.load().lvar_csp_attn_fwd(_view(q), _view(k), _view(v), _view(o_accum), _view(o), _ptr(M), _ptr(L),
+                                              indices.data_ptr(), counts.data_ptr(), G, indices.stride(2), bm,
+                                              B, H, Lq, Lk, d, float(o_scale), _scale(q, scale), _stream(q))
+        else:
+            st = _lib.load().lvar_csp_attn_upsample_fwd(
+                _view(q), _view(k), _view(v), _view(o_accum), int(upsample_from[0]), int(upsample_from[1]), _view(o),
+                _ptr(M), _ptr(L), indices.data_ptr(), counts.data_ptr(), G, indices.stride(2), bm,
+                B, H, Lq, Lk, d, float(o_scale), _scale(q, scale), _stream(q))
+    _lib.check(st, "lvar_csp_attn_fwd" if upsample_from is None else "lvar_csp_attn_upsample_fwd")
     return o, M, L
 
 
@@ -204,6 +216,22 @@ def csp_attn(q, k, v, scale, indices, indices_counts, o, o_scale):
              f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}, k: {tuple(k.shape)}")
     _require(tuple(o.shape) == tuple(q.shape), f"Output shape mismatch - o: {tuple(o.shape)}, q: {tuple(q.shape)}")
     out, _, _ = _csp_launch(q, k, v, indices, indices_counts, o, o_scale, scale, False)
+    return out
+
+
+def csp_attn_upsampled(q, k, v, scale, indices, indices_counts, o_cache, o_scale=1):
+    """Sparse step with the O-cache resampled inside the attention epilogue:
+    ``upsample(o_cache) + o_scale * softmax(q k[idx]^T scale) v[idx]`` where ``o_cache`` ``[B,H,h*h,d]``
+    is the cached output of a coarser ``h x h`` scale and the queries form an ``h' x h'`` grid
+    (``Lq = h'*h'``); the resampling is bilinear with half-pixel centres (``align_corners=False``).
+    One launch and one rounding for ``upsample_Ocache(...).to(v.dtype)`` followed by ``csp_attn``
+    (models/sparvar/sparse_attn.py:324-362, 1129-1142); the upsampled cache never goes to memory."""
+    _require(indices.dim() == 4 and indices.shape[-1] == k.shape[-2] and indices.shape[:2] == q.shape[:2],
+             f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}, k: {tuple(k.shape)}")
+    _require(o_cache.dim() == 4, "o_cache must be [B,H,h*h,d]")
+    src, dst = math.isqrt(o_cache.shape[-2]), math.isqrt(q.shape[-2])
+    _require(src * src == o_cache.shape[-2] and dst * dst == q.shape[-2], "o_cache and q must hold square token grids")
+    out, _, _ = _csp_launch(q, k, v, indices, indices_counts, o_cache, o_scale, scale, False, upsample_from=(src, dst))
     return out
 
 

@@ -72,9 +72,8 @@ class SparseDiffAttn:
             o = self.out_cache
             if o.shape[0] != q.shape[0]:
                 o = o[:q.shape[0]]
-            o = mb.upsample_ocache(o, o.shape[-2], q.shape[-2]).to(v.dtype)
-        else:
-            o = torch.zeros_like(q)
-        return ops.csp_attn(q, k, v, scale, inds, counts, o, 1)
+            # bilinear upsample of the cache fused into the attention epilogue (sparse_attn.py:1129-1142)
+            return ops.csp_attn_upsampled(q, k, v, scale, inds, counts, o, 1)
+        return ops.csp_attn(q, k, v, scale, inds, counts, torch.zeros_like(q), 1)
 
     __call__ = forward

@@ -163,3 +163,38 @@ def test_mask_to_lists_matches_oracle():
         cnt, idx = ops.mask_to_lists(m.cuda(), mult)
         e_cnt, e_idx = oracle.mask_to_lists(m, mult)
         assert torch.equal(cnt.cpu(), e_cnt) and torch.equal(idx.cpu(), e_idx), (shape, p, mult)
+
+
+@pytest.mark.gpu
+def test_csp_attn_with_fused_ocache_upsample():
+    """The sparse step with the O-cache resampled in the epilogue equals bilinear upsampling
+    (library F.interpolate, align_corners=False, and the oracle's closed form) followed by the
+    token-list attention; with empty lists it is the upsampling alone."""
+    import torch.nn.functional as F
+    import oracle
+    from lvar_amd import sparse_attn_ops as ops
+    g = torch.Generator().manual_seed(9)
+    for (src, dst, d, Lk, cnt) in ((5, 8, 128, 200, 64), (16, 20, 64, 521, 128), (40, 48, 128, 1500, 192), (3, 16, 128, 300, 0)):
+        B, H, Lq = 1, 2, dst * dst
+        q = (torch.randn(B, H, Lq, d, generator=g) * 0.5).to(torch.bfloat16)
+        k = (torch.randn(B, H, Lk, d, generator=g) * 0.5).to(torch.bfloat16)
+        v = (torch.randn(B, H, Lk, d, generator=g) * 0.5).to(torch.bfloat16)
+        cache = torch.randn(B, H, src * src, d, generator=g).to(torch.bfloat16)
+        G = (Lq + 191) // 192
+        idx = torch.zeros(B, H, G, Lk, dtype=torch.int32)
+        for b in range(B):
+            for h in range(H):
+                for gg in range(G):
+                    idx[b, h, gg, :cnt] = torch.randperm(Lk, generator=g)[:cnt].to(torch.int32)
+        counts = torch.full((B, H, G), cnt, dtype=torch.int32)
+        out = ops.csp_attn_upsampled(q.cuda(), k.cuda(), v.cuda(), None, idx.cuda(), counts.cuda(), cache.cuda(), 1)
+        up = oracle.upsample_ocache(cache, src * src, dst * dst)
+        lib = F.interpolate(cache.float().view(B * H, src, src, d).permute(0, 3, 1, 2), size=(dst, dst), mode="bilinear",
+                            align_corners=False).permute(0, 2, 3, 1).reshape(B, H, Lq, d)
+        assert torch.allclose(up.float(), lib, atol=1e-4)      # fp32 tap weights in the library routine
+        ref = oracle.csp_attn(q, k, v, None, idx, counts, up, 1)
+        assert close(out, ref), (src, dst, d)
+        if cnt == 0:
+            assert torch.allclose(out.float().cpu(), lib, atol=2e-2, rtol=1e-2)
+    with pytest.raises(AssertionError):
+        ops.csp_attn_upsampled(q.cuda(), k.cuda(), v.cuda(), None, idx.cuda(), counts.cuda(), cache[:, :, :8].cuda(), 1)
