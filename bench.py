@@ -181,19 +181,16 @@ def main():
             config.update({"block": [bq, bk], "mask": "sink(scales<=16)+window(+-2 blocks/scale)+colsum top-k", "density": 0.25})
         elif wl == "video_10":
             # 3D local window over a latent grid of 8 frames x 64 x 64 tokens (+-1 frame, +-1 spatial
-            # block) plus 2 % of blocks by colsum top-k of a strided query sample
+            # block of 128 tokens) plus colsum top-k blocks (scores from every 4th query row) up to 10 % density
             blk = torch.arange(nQ, device=dev)
-            f, s = blk // 32, blk % 32                                      # 32 blocks of 128 tokens per frame
-            near = ((f[:, None] - f[None, :]).abs() <= 1) & ((s[:, None] - s[None, :]).abs() <= 1)
-            cs = ops.colsum(qg[:, :, ::8].contiguous(), kg, scale, q_group_size=32)   # 4096 sampled rows, groups of 32
-            score = mb.key_block_sums(cs, bk)[:, :, :nQ]
-            score = score.masked_fill(near[None, None], -float("inf"))
-            extra = int(round(0.02 * nK))
-            top = torch.topk(score, k=extra, dim=-1).indices
-            mask = near[None, None].expand(B, H, nQ, nK).clone()
-            mask.scatter_(-1, top, True)
-            del cs, score
-            config.update({"block": [bq, bk], "mask": "3D window (+-1 frame, +-1 spatial block) + 2% colsum top-k"})
+            f, s_ = blk // 32, blk % 32                                     # 32 blocks of 128 tokens per frame
+            near = ((f[:, None] - f[None, :]).abs() <= 1) & ((s_[:, None] - s_[None, :]).abs() <= 1)
+            cs = ops.colsum(qg[:, :, ::4].contiguous(), kg, scale, q_group_size=32)   # every 4th query row: 32 samples per 128-row block
+            score = mb.key_block_sums(cs, bk)[:, :, :nQ].contiguous()
+            del cs
+            num, idx = ops.block_topk_lists(score, int(round(0.10 * nK)), near)
+            mask = None
+            config.update({"block": [bq, bk], "mask": "3D window (+-1 frame, +-1 spatial block) + colsum top-k blocks up to 10 %"})
         else:
             pct = float(wl.split("_")[1])
             g = torch.Generator().manual_seed(7)
@@ -201,9 +198,10 @@ def main():
             mask.scatter_(-1, torch.randint(0, nK, (B, H, nQ, 1), generator=g), True)
             mask = mask.to(dev)
             config.update({"block": [bq, bk], "mask": f"Bernoulli({pct}%) blocks, >=1 per row"})
-        num, idx = mb.block_mask_to_lists(mask)
+        if mask is not None:
+            num, idx = mb.block_mask_to_lists(mask)
         flops = block_flops(num, idx, Lq, Lk, d, bq, bk, B, H)
-        config["active_block_fraction"] = round(float(mask.float().mean().item()), 4)
+        config["active_block_fraction"] = round(float(num.float().mean().item()) / nK, 4)
         fn = lambda: ops.block_sparse_attn(qg, kg, vg, num, idx, bq, bk, scale)
         kernel = "attn_fwd_kernel<128,4,MODE_BLOCK>"
         if not args.no_cpu_baseline:
@@ -230,9 +228,15 @@ def main():
     elif wl == "csp":
         G = (Lq + 191) // 192
         cs = ops.colsum(qg, kg, scale)
-        inds, counts = mb.topk_index_list(cs, 0.2)
-        del cs
+        inds, counts = mb.topk_index_list(cs, 0.2, order="index")     # GPU radix select, ascending key order
         cnt = int(counts[0, 0, 0])
+        if not args.no_aux:
+            topk_ms, _ = time_launches(lambda: ops.topk_token_lists(cs, cnt), 10, 3)
+            torch_ms, _ = time_launches(lambda: torch.topk(cs, cnt, dim=-1), 5, 2)
+            ref_set = torch.topk(cs, cnt, dim=-1).indices.sort(-1).values
+            assert torch.equal(inds[..., :cnt].long(), ref_set), "GPU top-k set differs from torch.topk"
+            aux = {"topk_token_lists_us": round(topk_ms * 1e3, 1), "torch_topk_us": round(torch_ms * 1e3, 1)}
+        del cs
         rows = torch.tensor([min(192, Lq - g * 192) for g in range(G)], dtype=torch.float64)
         flops = 4.0 * d * B * H * float(rows.sum()) * cnt
         o0 = torch.zeros_like(qg)

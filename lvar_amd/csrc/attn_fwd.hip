@@ -516,12 +516,8 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
   p.total_wg = p.B * p.H * p.nqt;
   const int grid = ((p.total_wg + 7) / 8) * 8;
   auto kern = attn_fwd_kernel<D, NWAVES, MODE, ACCUM, LSE_ONLY>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != hipSuccess)
-      return LVAR_ELAUNCH;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ready{0};
+  if (!ensure_lds_limit((const void*)kern, SMEM, lds_ready)) return LVAR_ELAUNCH;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(NWAVES * 64), SMEM, stream, p);
   return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
 }

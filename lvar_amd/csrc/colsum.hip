@@ -223,12 +223,8 @@ static int launch_cs(const ColsumParams& p0, hipStream_t stream) {
   p.total_wg = p.B * p.H * p.nkt;
   const int grid = ((p.total_wg + 7) / 8) * 8;
   constexpr int SMEM = 4 * 64 * D * 2 + 8 * 256;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)colsum_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != hipSuccess)
-      return LVAR_ELAUNCH;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ready{0};
+  if (!ensure_lds_limit((const void*)colsum_kernel<D>, SMEM, lds_ready)) return LVAR_ELAUNCH;
   hipLaunchKernelGGL((colsum_kernel<D>), dim3(grid), dim3(256), SMEM, stream, p);
   return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
 }

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include "common.h"
 #include "../../include/lvar_sparse_attn.h"
 
@@ -80,6 +81,18 @@ struct MaskCompactParams {
   int64_t mask_stride, out_stride;
   int rows, n, out_len, multiple_of, zero_tail;
 };
+
+// Raises a kernel's dynamic-LDS limit once per device (the attribute is kept per device); `done` is a
+// per-kernel bit set of the devices already handled.  Safe to call from several host threads.
+inline bool ensure_lds_limit(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+  done.fetch_or(bit, std::memory_order_release);
+  return true;
+}
 
 int launch_topk_token_lists(const TopkListParams& p, hipStream_t s);
 int launch_remap_concat_lists(const RemapListParams& p, hipStream_t s);
