@@ -117,13 +117,72 @@ def cpu_baseline_dense(q, k, v, budget_s=20.0, colsum=False):
     return done, t_used
 
 
+def run_infinity_schedule(args, dev):
+    """Attention time of one Infinity-2B 1024^2 image (13 scales x 32 layers, B=2 for classifier-free
+    guidance, H16 d128): every layer dense, against the SparVAR schedule of the reference's shipped
+    configuration (models/sparvar/sparse-attn-config.yml:15-34): scales 0-9 dense; scales 10-12:
+    layers 0-10 column-sparse (full step at scale 10, sparse steps with the upsampled O-cache at 11 and
+    12), layers 11-31 sink + local-window block masks.  One layer of every distinct shape is timed and
+    multiplied by its layer count."""
+    from lvar_amd import mask_build as mb
+    from lvar_amd import sparse_attn_config as cfg
+    from lvar_amd import sparse_attn_ops as ops
+    from lvar_amd.sparse_diff_attn import SparseDiffAttn
+    from lvar_amd.sparse_flex_attn import SparseFlexAttn
+    scales = list(mb.INFINITY_SCALES)
+    offs = mb.scale_offsets(scales)
+    B, H, d, n_layers, bound = 2, 16, 128, 32, 10
+    win = [-1, -1, -1, -1, -1, -1, -1, -1, 1, 1, 3, 5, 7]
+    cfg.reset()
+    cfg.GLOBAL_CONFIG["attn"]["top_keys"] = 0.2                        # the shipped value (sparse-attn-config.yml:19)
+    steps, warm = max(5, args.steps // 5), max(3, args.warmup // 4)
+    g = torch.Generator().manual_seed(99)
+    mk = lambda L: (torch.randn(B, H, L, d, generator=g) * 0.5).to(torch.bfloat16).to(dev)
+    dense_ms, sparse_ms, rows = 0.0, 0.0, []
+    diff = SparseDiffAttn(scales=scales, spsd_scale=10)
+    for si, S in enumerate(scales):
+        Lq, Lk = S * S, offs[si + 1]
+        q, k, v = mk(Lq), mk(Lk), mk(Lk)
+        t_dense, _ = time_launches(lambda: ops.dense_attn(q, k, v, None), steps, warm)
+        dense_ms += n_layers * t_dense
+        if si < 10:
+            sparse_ms += n_layers * t_dense
+            rows.append({"scale": S, "Lq": Lq, "Lk": Lk, "dense_us": round(t_dense * 1e3, 1)})
+            continue
+        flex = SparseFlexAttn([(s, s) for s in scales], win, q_scale_idx=si, attn_sink_scale=5, num_heads=H, device=dev)
+        t_flex, _ = time_launches(lambda: flex(q, k, v, None), steps, warm)
+        if si == 10:
+            t_cs4a, _ = time_launches(lambda: diff(q, k, v, None, do_full_step=True, scale_ind=si), steps, warm)
+        else:
+            saved = (diff.indices, diff.counts, diff.count_host)
+
+            def sparse_step():
+                diff.indices, diff.counts, diff.count_host = saved      # every timed call starts from the same cached lists
+                return diff(q, k, v, None, scale_ind=si)
+            t_cs4a, _ = time_launches(sparse_step, steps, warm)
+            diff.indices, diff.counts, diff.count_host = saved
+            diff(q, k, v, None, scale_ind=si)                             # leaves the lists of this scale for the next one
+        sparse_ms += (bound + 1) * t_cs4a + (n_layers - bound - 1) * t_flex
+        rows.append({"scale": S, "Lq": Lq, "Lk": Lk, "dense_us": round(t_dense * 1e3, 1), "cs4a_layer_us": round(t_cs4a * 1e3, 1),
+                     "csla_layer_us": round(t_flex * 1e3, 1), "csla_block_density": round(flex.density, 4)})
+    print(json.dumps({
+        "metric": "self-attention time per Infinity-2B 1024^2 image (all scales, 32 layers), SparVAR schedule", "value": round(sparse_ms, 3),
+        "unit": "ms", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(sparse_ms, 3), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic (seeded N(0,1)*0.5, random-init, no checkpoint)",
+        "config": {"workload": "infinity2b_schedule", "B": B, "H": H, "head_dim": d, "layers": n_layers, "scales": scales,
+                   "decision_scale": 10, "top_keys": cfg.GLOBAL_CONFIG["attn"]["top_keys"], "bound_layer": bound, "attn_sink": 5, "win_size": win},
+        "all_dense_ms": round(dense_ms, 3), "speedup_vs_all_dense": round(dense_ms / sparse_ms, 3), "per_scale": rows,
+        "device": torch.cuda.get_device_name(0)}))
+    cfg.reset()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="block_sparse_25",
-                    help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | density_<pct> | video_10 | copy_1gib")
+                    help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | density_<pct> | video_10 | infinity2b_schedule | copy_1gib")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aux", action="store_true", help="skip the companion dense/colsum/mask-build timings")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0)
@@ -143,6 +202,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     wl = args.workload
+    if wl == "infinity2b_schedule":
+        run_infinity_schedule(args, dev)
+        return
     if wl == "copy_1gib":
         # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         x = torch.empty(1 << 28, dtype=torch.float32, device=dev)

@@ -41,6 +41,9 @@ def _scale(q: torch.Tensor, scale) -> float:
 
 
 def _prep(t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dtype is torch.bfloat16 and t.is_cuda and t.dim() == 4 and t.is_contiguous() and t.shape[-1] % 8 == 0 \
+            and t.data_ptr() % 16 == 0:
+        return t                                   # the common case, checked without walking the strides
     _require(t.dim() == 4, f"{name} must be [B,H,L,d], got {tuple(t.shape)}")
     if t.dtype != torch.bfloat16:
         raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
@@ -77,8 +80,9 @@ def _dense_launch(q, k, v, scale, want_o=True, want_ml=True, want_lse2=False):
     B, H, Lq, d = q.shape
     Lk = k.shape[2]
     o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device) if want_o else None
-    M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device) if want_ml else None
-    L = torch.empty_like(M) if want_ml else None
+    M = L = None
+    if want_ml:
+        M, L = torch.empty((2, B, H, Lq, 1), dtype=torch.float32, device=q.device).unbind(0)   # one allocation
     lse2 = torch.empty((B, H, Lq), dtype=torch.float32, device=q.device) if want_lse2 else None
     with torch.cuda.device(q.device):
         st = _lib.load().lvar_dense_attn_fwd(_view(q), _view(k), _view(v if want_o else None), _view(o), _ptr(M), _ptr(L),
