@@ -198,3 +198,44 @@ def test_csp_attn_with_fused_ocache_upsample():
             assert torch.allclose(out.float().cpu(), lib, atol=2e-2, rtol=1e-2)
     with pytest.raises(AssertionError):
         ops.csp_attn_upsampled(q.cuda(), k.cuda(), v.cuda(), None, idx.cuda(), counts.cuda(), cache[:, :, :8].cuda(), 1)
+
+
+@pytest.mark.gpu
+def test_ops_replay_correctly_from_a_hip_graph():
+    """Every entry point only enqueues kernels on the caller's stream (no allocation, memset or
+    synchronisation inside the library), so a decision-scale step can be captured once and replayed.
+    Replays are interleaved with eager work and each one is compared with the eager result."""
+    from lvar_amd import sparse_attn_ops as ops
+    q, k, v = make_qkv(1, 2, 400, 921, 128, seed=21, amp=0.5)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+
+    def step():
+        o, cs, (M, L) = ops.dense_colsum_attn(qg, kg, vg)
+        inds, counts = ops.topk_token_lists(cs, 192)
+        cache = ops.csp_attn(qg, kg, vg, None, inds, counts, o, -1)
+        _, bsum = ops.colsum(qg, kg, None, q_group_size=128, lse=(M, L), return_block_sums=True)
+        num, idx = ops.block_topk_lists(bsum, 6)
+        ob, _ = ops.block_sparse_attn(qg, kg, vg, num, idx, 128, 64)
+        return o, cs, inds, cache, num, idx, ob
+
+    eager = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()                                                        # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for rep in range(3):
+        qg.add_(0)                                                        # eager work between replays
+        _ = ops.dense_attn(qg, kg, vg)
+        torch.cuda.synchronize()
+        for t in outs:
+            t.zero_()                                                     # a replay must rewrite every output
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, eager):
+            assert torch.equal(a, b), rep
