@@ -69,13 +69,6 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const int bh = w / p.nqt, qt = w - bh * p.nqt;
   const int b = bh / p.H, h = bh - b * p.H;
   const int tid = threadIdx.x, lane = tid & 63;
-#ifdef LVAR_ALT_PRIO
-  {
-    const int slot = __builtin_amdgcn_s_getreg(63492) & 1;  // hardware wave slot parity
-    const int round = (blockIdx.x / 512) & 1;
-    if (slot ^ round) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
-  }
-#endif
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, r = lane & 31;
   const int q0 = qt * WGROWS;
@@ -86,12 +79,20 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const bool identity = (MODE == MODE_BLOCK) && p.list == nullptr;
   const int32_t* list = nullptr;
   int T, count;
+  // first four entries of a block list, read together with the count (not after it): one memory
+  // round trip less before the first tile can be fetched; entries beyond the count are never used
+  int head[4] = {0, 0, 0, 0};
   if (identity) {
     count = (p.Lk + 63) >> 6;
     T = count;
   } else {
-    count = max(0, min(p.cnt[b * p.cnt_sb + h * p.cnt_sh + g], p.list_len));
     list = p.list + b * p.list_sb + h * p.list_sh + (int64_t)g * p.list_sg;
+    if (MODE == MODE_BLOCK) {
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        if (i < p.list_len) head[i] = list[i];
+    }
+    count = max(0, min(p.cnt[b * p.cnt_sb + h * p.cnt_sh + g], p.list_len));
     T = (MODE == MODE_BLOCK) ? (count << p.sub_shift) : ((count + 63) >> 6);
   }
   const int sub_shift = identity ? 0 : p.sub_shift;
@@ -279,11 +280,20 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     int nv0, nv1 = 64, nv2 = 64, nv3 = 64;
     {
       int rows0[NR];
-      prefetch_raw(0, raw);
+      // tiles 0..3: block lists use the entries read next to the count
+      auto first_raw = [&](int t, int (&raw)[NR]) {
+        if (MODE == MODE_BLOCK && !identity) {
+          const int e = t >> sub_shift;
+          raw[0] = (e == 0) ? head[0] : (e == 1) ? head[1] : (e == 2) ? head[2] : head[3];
+        } else {
+          prefetch_raw(t, raw);
+        }
+      };
+      first_raw(0, raw);
       finish_rows(0, raw, rows0, nv0);
-      if (T > 1) { prefetch_raw(1, raw); finish_rows(1, raw, rows_v, nv1); }
-      if (T > 2) { prefetch_raw(2, raw); finish_rows(2, raw, rows_k, nv2); }
-      if (T > 3) prefetch_raw(3, raw);
+      if (T > 1) { first_raw(1, raw); finish_rows(1, raw, rows_v, nv1); }
+      if (T > 2) { first_raw(2, raw); finish_rows(2, raw, rows_k, nv2); }
+      if (T > 3) first_raw(3, raw);
       issue(krsrc, k_srb, false, rows0, lds0);
       if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows0, lds0 + 2 * TILE);
       if (T > 1) issue(krsrc, k_srb, false, rows_v, lds0 + TILE);
