@@ -18,8 +18,8 @@ __device__ __forceinline__ int lanes_below(unsigned long long bal, int lane) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Exact top-k per row by radix select.  One 256-thread workgroup per row; wave w owns the w-th
-// contiguous quarter of the (padded) row and every thread keeps its KPT keys in registers (KPT = 0:
+// Exact top-k per row by radix select.  One 512-thread workgroup per row; wave w owns the w-th
+// contiguous eighth of the (padded) row and every thread keeps its KPT keys in registers (KPT = 0:
 // rows too long for that are re-read from L2 in every pass).
 //   3 histogram passes (11, 11 and 10 bits, most significant first; LDS atomics) narrow the k-th
 //   largest key down to its exact value T and the number `need` of keys equal to T that belong to
@@ -29,12 +29,13 @@ __device__ __forceinline__ int lanes_below(unsigned long long bal, int lane) {
 // ---------------------------------------------------------------------------------------------
 constexpr int TOPK_BINS = 2048;
 
-template <int KPT>
-__global__ __launch_bounds__(256) void topk_token_lists_kernel(const TopkListParams p) {
+template <int KPT, int NT>
+__global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kernel(const TopkListParams p) {
+  constexpr int NW = NT / 64;
   __shared__ int hist[TOPK_BINS];
-  __shared__ int wsum[4];
+  __shared__ int wsum[NW];
   __shared__ int sel[2];  // chosen bin, keys still wanted inside it
-  __shared__ int wgt[4], weq[4];
+  __shared__ int wgt[NW], weq[NW];
   const int row = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* s = p.scores + (int64_t)row * p.score_stride;
@@ -45,7 +46,7 @@ __global__ __launch_bounds__(256) void topk_token_lists_kernel(const TopkListPar
   if (want == 0) return;
 
   // chunk c of wave w covers columns (w * cpw + c) * 64 .. +63
-  const int cpw = KPT ? KPT : ((n + 255) >> 8);
+  const int cpw = KPT ? KPT : ((n + NT - 1) / NT);
   const int col0 = wave * cpw * 64 + lane;
   uint32_t keys[KPT ? KPT : 1];
   if (KPT) {
@@ -74,17 +75,17 @@ __global__ __launch_bounds__(256) void topk_token_lists_kernel(const TopkListPar
     const int shift = (pass == 0) ? 21 : (pass == 1) ? 10 : 0;
     const int bits = (pass == 2) ? 10 : 11;
     const int nbins = 1 << bits;
-    for (int t = tid; t < nbins; t += 256) hist[t] = 0;
+    for (int t = tid; t < nbins; t += NT) hist[t] = 0;
     __syncthreads();
     visit([&](int j, uint32_t key) {
       if (j < n && (key & pmask) == prefix) atomicAdd(&hist[(key >> shift) & (nbins - 1)], 1);
     });
     __syncthreads();
     // thread t owns the bpt bins nbins-1 - t*bpt .. (descending); find the bin holding the want-th key from the top
-    const int bpt = nbins >> 8;
+    const int bpt = (nbins + NT - 1) / NT;   // 1 when there are as many threads as bins (then every thread owns one)
     const int btop = nbins - 1 - tid * bpt;
     int mine = 0;
-    for (int e = 0; e < bpt; e++) mine += hist[btop - e];
+    for (int e = 0; e < bpt; e++) mine += (btop - e >= 0) ? hist[btop - e] : 0;
     int incl = mine;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(256) void topk_token_lists_kernel(const TopkListPar
     if (before < want && want <= before + mine) {  // exactly one thread
       int acc = before, bin = btop;
       for (int e = 0; e < bpt; e++) {
-        const int h = hist[btop - e];
+        const int h = (btop - e >= 0) ? hist[btop - e] : 0;
         if (acc + h >= want) { bin = btop - e; break; }
         acc += h;
       }
@@ -140,13 +141,14 @@ __global__ __launch_bounds__(256) void topk_token_lists_kernel(const TopkListPar
 
 int launch_topk_token_lists(const TopkListParams& p, hipStream_t stream) {
   if (p.rows == 0) return LVAR_OK;
-  const dim3 grid(p.rows), block(256);
-  if (p.n <= 256 * 8) hipLaunchKernelGGL(topk_token_lists_kernel<8>, grid, block, 0, stream, p);
-  else if (p.n <= 256 * 16) hipLaunchKernelGGL(topk_token_lists_kernel<16>, grid, block, 0, stream, p);
-  else if (p.n <= 256 * 32) hipLaunchKernelGGL(topk_token_lists_kernel<32>, grid, block, 0, stream, p);
-  else if (p.n <= 256 * 48) hipLaunchKernelGGL(topk_token_lists_kernel<48>, grid, block, 0, stream, p);
-  else if (p.n <= 256 * 64) hipLaunchKernelGGL(topk_token_lists_kernel<64>, grid, block, 0, stream, p);
-  else hipLaunchKernelGGL(topk_token_lists_kernel<0>, grid, block, 0, stream, p);
+  const dim3 grid(p.rows);
+  // 512 threads per row keep a row of up to 16384 keys in registers (KPT keys per thread)
+  if (p.n <= 512 * 4) hipLaunchKernelGGL((topk_token_lists_kernel<4, 512>), grid, dim3(512), 0, stream, p);
+  else if (p.n <= 512 * 8) hipLaunchKernelGGL((topk_token_lists_kernel<8, 512>), grid, dim3(512), 0, stream, p);
+  else if (p.n <= 512 * 16) hipLaunchKernelGGL((topk_token_lists_kernel<16, 512>), grid, dim3(512), 0, stream, p);
+  else if (p.n <= 512 * 24) hipLaunchKernelGGL((topk_token_lists_kernel<24, 512>), grid, dim3(512), 0, stream, p);
+  else if (p.n <= 512 * 32) hipLaunchKernelGGL((topk_token_lists_kernel<32, 512>), grid, dim3(512), 0, stream, p);
+  else hipLaunchKernelGGL((topk_token_lists_kernel<0, 512>), grid, dim3(512), 0, stream, p);
   return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
 }
 
