@@ -78,6 +78,18 @@ def time_launches(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall * 1e3 / steps
 
 
+def per_launch_stats(fn, n=50):
+    """Median and minimum duration of single launches (one event pair per launch, same stream)."""
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    t = sorted(a.elapsed_time(b) for a, b in evs)
+    return {"median_ms": round(t[len(t) // 2], 5), "min_ms": round(t[0], 5), "launches": n}
+
+
 def cpu_baseline_block_sparse(q, k, v, num, idx, bq, bk, budget_s=20.0):
     """Oracle (torch fp32 on the host cores) on a bounded sample of the same workload: whole
     (batch, head) slices until ~budget_s of CPU time is spent.  Returns TFLOP/s and a description."""
@@ -310,6 +322,7 @@ def main():
 
     ms, wall_ms = time_launches(fn, args.steps, args.warmup)
     tflops = flops / (ms * 1e-3) / 1e12
+    single = per_launch_stats(fn)
 
     if wl == "block_sparse_25" and not args.no_aux:
         # companion numbers named by the metric: colsum (+ mask build) versus the dense attention it replaces
@@ -340,7 +353,8 @@ def main():
         "config": config,
         "roofline": {"bound": "mfma", "kernel": kernel, "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC.get(wl),
-                     "flops_per_launch": flops, "host_wall_ms_per_step": round(wall_ms, 5)},
+                     "flops_per_launch": flops, "host_wall_ms_per_step": round(wall_ms, 5),
+                     "single_launch": single, "cache_state": "warm: back-to-back launches on the same inputs, no L2 flush"},
         "cpu_baseline": cpu,
         "device": torch.cuda.get_device_name(0),
     }
