@@ -31,9 +31,11 @@ class ShapeError(AssertionError, ValueError):
     """Shape / dtype contract violation (the reference raises AssertionError at the same places)."""
 
 
-def _require(cond: bool, msg: str) -> None:
+def _require(cond: bool, msg) -> None:
+    """``msg`` is a string or a zero-argument callable that builds it (so that hot paths do not
+    format messages that are never shown)."""
     if not cond:
-        raise ShapeError(msg)
+        raise ShapeError(msg() if callable(msg) else msg)
 
 
 def _scale(q: torch.Tensor, scale) -> float:
@@ -44,7 +46,7 @@ def _prep(t: torch.Tensor, name: str) -> torch.Tensor:
     if t.dtype is torch.bfloat16 and t.is_cuda and t.dim() == 4 and t.is_contiguous() and t.shape[-1] % 8 == 0 \
             and t.data_ptr() % 16 == 0:
         return t                                   # the common case, checked without walking the strides
-    _require(t.dim() == 4, f"{name} must be [B,H,L,d], got {tuple(t.shape)}")
+    _require(t.dim() == 4, lambda: f"{name} must be [B,H,L,d], got {tuple(t.shape)}")
     if t.dtype != torch.bfloat16:
         raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
     if not t.is_cuda:
@@ -61,15 +63,45 @@ def _view(t: Optional[torch.Tensor]) -> _lib.LvarTensor:
 
 
 def _check_qkv(q, k, v):
-    _require(k.shape == v.shape, f"k/v shape mismatch: {tuple(k.shape)} vs {tuple(v.shape)}")
-    _require(q.shape[0] == k.shape[0] and q.shape[1] == k.shape[1] and q.shape[3] == k.shape[3],
-             f"q/k batch, head or head_dim mismatch: {tuple(q.shape)} vs {tuple(k.shape)}")
-    _require(q.shape[-1] in (64, 128), f"head_dim must be 64 or 128, got {q.shape[-1]}")
-    _require(q.device == k.device == v.device, "q, k, v must be on the same device")
+    # messages are only formatted on failure: these checks run on every call
+    qs, ks = q.shape, k.shape
+    if ks != v.shape:
+        raise ShapeError(f"k/v shape mismatch: {tuple(k.shape)} vs {tuple(v.shape)}")
+    if qs[0] != ks[0] or qs[1] != ks[1] or qs[3] != ks[3]:
+        raise ShapeError(f"q/k batch, head or head_dim mismatch: {tuple(q.shape)} vs {tuple(k.shape)}")
+    if qs[3] != 128 and qs[3] != 64:
+        raise ShapeError(f"head_dim must be 64 or 128, got {q.shape[-1]}")
+    if not (q.device == k.device == v.device):
+        raise ShapeError("q, k, v must be on the same device")
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream(t: torch.Tensor) -> int:
+    """Raw handle of torch's current stream on the tensor's device."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _on_device:
+    """``with _on_device(t):`` makes the tensor's device current for the launch, and does nothing
+    (no guard object, no runtime calls) when it already is."""
+    __slots__ = ("guard",)
+
+    def __init__(self, t: torch.Tensor):
+        idx = t.device.index
+        self.guard = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(idx)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -84,7 +116,7 @@ def _dense_launch(q, k, v, scale, want_o=True, want_ml=True, want_lse2=False):
     if want_ml:
         M, L = torch.empty((2, B, H, Lq, 1), dtype=torch.float32, device=q.device).unbind(0)   # one allocation
     lse2 = torch.empty((B, H, Lq), dtype=torch.float32, device=q.device) if want_lse2 else None
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         st = _lib.load().lvar_dense_attn_fwd(_view(q), _view(k), _view(v if want_o else None), _view(o), _ptr(M), _ptr(L),
                                             _ptr(lse2), B, H, Lq, Lk, d, _scale(q, scale), _stream(q))
     _lib.check(st, "lvar_dense_attn_fwd")
@@ -111,7 +143,7 @@ def _colsum_given_lse(q, k, lse2, scale, q_group_size, want_block_sums=False):
     G = (Lq + q_group_size - 1) // q_group_size
     cs = torch.empty((B, H, G, Lk), dtype=torch.float32, device=q.device)
     bs = torch.empty((B, H, G, (Lk + 63) // 64), dtype=torch.float32, device=q.device) if want_block_sums else None
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         st = _lib.load().lvar_colsum_fwd(_view(q), _view(k), lse2.data_ptr(), cs.data_ptr(), _ptr(bs),
                                         B, H, Lq, Lk, d, q_group_size, _scale(q, scale), _stream(q))
     _lib.check(st, "lvar_colsum_fwd")
@@ -173,11 +205,11 @@ def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, u
     Lk = k.shape[2]
     bm = get_kernel_config_attn()["bm"]
     _require(indices.dim() == 4 and indices.shape[0] == B and indices.shape[1] == H,
-             f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}")
+             lambda: f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}")
     G = indices.shape[2]
-    _require(G * bm >= Lq, f"indices has {G} query groups of {bm} rows, fewer than Lq={Lq}")
+    _require(G * bm >= Lq, lambda: f"indices has {G} query groups of {bm} rows, fewer than Lq={Lq}")
     _require(tuple(counts.shape) == tuple(indices.shape[:-1]),
-             f"Indices counts shape mismatch - indices_counts: {tuple(counts.shape)}, indices: {tuple(indices.shape)}")
+             lambda: f"Indices counts shape mismatch - indices_counts: {tuple(counts.shape)}, indices: {tuple(indices.shape)}")
     if indices.dtype != torch.int32 or counts.dtype != torch.int32:
         raise TypeError("indices and indices_counts must be int32")
     _require(indices.device == q.device and counts.device == q.device, "indices / counts must be on q's device")
@@ -187,18 +219,18 @@ def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, u
     if o_accum is not None:
         o_accum = _prep(o_accum, "o")
         if upsample_from is None:
-            _require(o_accum.shape == q.shape, f"Output shape mismatch - o: {tuple(o_accum.shape)}, q: {tuple(q.shape)}")
+            _require(o_accum.shape == q.shape, lambda: f"Output shape mismatch - o: {tuple(o_accum.shape)}, q: {tuple(q.shape)}")
         else:
             src, dst = upsample_from
             _require(dst * dst == Lq and tuple(o_accum.shape) == (B, H, src * src, d),
-                     f"O-cache shape mismatch - o_cache: {tuple(o_accum.shape)}, expected {(B, H, src * src, d)} "
+                     lambda: f"O-cache shape mismatch - o_cache: {tuple(o_accum.shape)}, expected {(B, H, src * src, d)} "
                      f"for a {src}x{src} -> {dst}x{dst} grid, q: {tuple(q.shape)}")
     o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device)
     M = L = None
     if want_stats:
         M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
         L = torch.empty_like(M)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         if upsample_from is None:
             st = _lib.load().lvar_csp_attn_fwd(_view(q), _view(k), _view(v), _view(o_accum), _view(o), _ptr(M), _ptr(L),
                                               indices.data_ptr(), counts.data_ptr(), G, indices.stride(2), bm,
@@ -217,8 +249,8 @@ def csp_attn(q, k, v, scale, indices, indices_counts, o, o_scale):
     (reference ``csp_attn``, sparse_attn_ops.py:273-292).  Returns a new tensor; ``o`` is not
     modified (the reference's Triton behaviour).  The sum is formed in fp32 and rounded once."""
     _require(indices.dim() == 4 and indices.shape[-1] == k.shape[-2] and indices.shape[:2] == q.shape[:2],
-             f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}, k: {tuple(k.shape)}")
-    _require(tuple(o.shape) == tuple(q.shape), f"Output shape mismatch - o: {tuple(o.shape)}, q: {tuple(q.shape)}")
+             lambda: f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}, k: {tuple(k.shape)}")
+    _require(tuple(o.shape) == tuple(q.shape), lambda: f"Output shape mismatch - o: {tuple(o.shape)}, q: {tuple(q.shape)}")
     out, _, _ = _csp_launch(q, k, v, indices, indices_counts, o, o_scale, scale, False)
     return out
 
@@ -231,7 +263,7 @@ def csp_attn_upsampled(q, k, v, scale, indices, indices_counts, o_cache, o_scale
     One launch and one rounding for ``upsample_Ocache(...).to(v.dtype)`` followed by ``csp_attn``
     (models/sparvar/sparse_attn.py:324-362, 1129-1142); the upsampled cache never goes to memory."""
     _require(indices.dim() == 4 and indices.shape[-1] == k.shape[-2] and indices.shape[:2] == q.shape[:2],
-             f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}, k: {tuple(k.shape)}")
+             lambda: f"Indices shape mismatch - indices: {tuple(indices.shape)}, q: {tuple(q.shape)}, k: {tuple(k.shape)}")
     _require(o_cache.dim() == 4, "o_cache must be [B,H,h*h,d]")
     src, dst = math.isqrt(o_cache.shape[-2]), math.isqrt(q.shape[-2])
     _require(src * src == o_cache.shape[-2] and dst * dst == q.shape[-2], "o_cache and q must hold square token grids")
@@ -259,7 +291,7 @@ def block_sparse_attn(q, k, v, kv_num_blocks, kv_indices, block_q: int = 128, bl
     nQ = (Lq + block_q - 1) // block_q
     _require(kv_num_blocks.dim() == 3 and kv_indices.dim() == 4, "kv_num_blocks must be [B,H,nQ], kv_indices [B,H,nQ,nKmax]")
     _require(kv_num_blocks.shape[2] == nQ and kv_indices.shape[2] == nQ,
-             f"block list has {kv_num_blocks.shape[2]} query blocks, expected {nQ}")
+             lambda: f"block list has {kv_num_blocks.shape[2]} query blocks, expected {nQ}")
     _require(kv_num_blocks.shape[0] in (1, B) and kv_num_blocks.shape[1] in (1, H)
              and tuple(kv_indices.shape[:2]) == tuple(kv_num_blocks.shape[:2]), "block list batch/head dims must be 1 or B/H")
     if kv_num_blocks.dtype != torch.int32 or kv_indices.dtype != torch.int32:
@@ -273,7 +305,7 @@ def block_sparse_attn(q, k, v, kv_num_blocks, kv_indices, block_q: int = 128, bl
     o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device)
     M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
     L = torch.empty_like(M)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         st = _lib.load().lvar_block_sparse_attn_fwd(
             _view(q), _view(k), _view(v), _view(o), M.data_ptr(), L.data_ptr(),
             kv_num_blocks.data_ptr(), nb_sb, nb_sh, kv_indices.data_ptr(), ki_sb, ki_sh, kv_indices.stride(2), kv_indices.shape[3],
@@ -295,11 +327,11 @@ def block_topk_lists(block_scores, target: int, base_mask=None):
     _require(nK <= 2048, "at most 2048 key blocks per row")
     base = None
     if base_mask is not None:
-        _require(tuple(base_mask.shape) == (nQ, nK), f"base_mask must be [nQ,nK] = {(nQ, nK)}")
+        _require(tuple(base_mask.shape) == (nQ, nK), lambda: f"base_mask must be [nQ,nK] = {(nQ, nK)}")
         base = base_mask.to(device=bs.device, dtype=torch.uint8).contiguous()
     num = torch.empty((B, H, nQ), dtype=torch.int32, device=bs.device)
     idx = torch.empty((B, H, nQ, nK), dtype=torch.int32, device=bs.device)
-    with torch.cuda.device(bs.device):
+    with _on_device(bs):
         st = _lib.load().lvar_block_topk_lists(bs.data_ptr(), _ptr(base), num.data_ptr(), idx.data_ptr(),
                                               B, H, nQ, nK, int(target), _stream(bs))
     _lib.check(st, "lvar_block_topk_lists")
@@ -322,12 +354,12 @@ def topk_token_lists(scores, k: int, out_len: Optional[int] = None, order: str =
     Lk = sc.shape[-1]
     rows = sc.numel() // Lk if Lk else 0
     k = int(k)
-    _require(0 <= k <= Lk, f"k = {k} must lie in [0, Lk = {Lk}]")
+    _require(0 <= k <= Lk, lambda: f"k = {k} must lie in [0, Lk = {Lk}]")
     out_len = Lk if out_len is None else int(out_len)
     _require(out_len >= k, "out_len must be at least k")
     idx = torch.zeros(sc.shape[:-1] + (out_len,), dtype=torch.int32, device=sc.device)
     cnt = torch.empty(sc.shape[:-1], dtype=torch.int32, device=sc.device)
-    with torch.cuda.device(sc.device):
+    with _on_device(sc):
         st = _lib.load().lvar_topk_token_lists(sc.data_ptr(), Lk, idx.data_ptr(), out_len, cnt.data_ptr(),
                                               rows, Lk, k, _stream(sc))
     _lib.check(st, "lvar_topk_token_lists")
@@ -359,14 +391,14 @@ def remap_concat_lists(src_indices, src_count: int, cur_q_len: int, cur_k_len: i
     L = 0
     loc = None
     if local_indices is not None:
-        _require(local_indices.dim() == 2 and local_indices.shape[0] == Gk, f"local_indices must be [Gk = {Gk}, L]")
+        _require(local_indices.dim() == 2 and local_indices.shape[0] == Gk, lambda: f"local_indices must be [Gk = {Gk}, L]")
         loc = local_indices.to(device=src.device, dtype=torch.int64).contiguous()
         L = loc.shape[1]
     out_len = int(cur_k_len) if out_len is None else int(out_len)
-    _require(cnt + L <= out_len, f"list length {cnt + L} exceeds the output width {out_len}")
+    _require(cnt + L <= out_len, lambda: f"list length {cnt + L} exceeds the output width {out_len}")
     out = torch.zeros((B, H, Gk, out_len), dtype=torch.int32, device=src.device)
     counts = torch.empty((B, H, Gk), dtype=torch.int32, device=src.device)
-    with torch.cuda.device(src.device):
+    with _on_device(src):
         st = _lib.load().lvar_remap_concat_lists(src.data_ptr(), Ks, Ks, _ptr(loc), L, L, out.data_ptr(), out_len,
                                                 counts.data_ptr(), B * H, Gs, Gk, cnt, int(cur_k_len), _stream(src))
     _lib.check(st, "lvar_remap_concat_lists")
@@ -386,7 +418,7 @@ def mask_to_lists(mask, multiple_of: int = 1):
     rows = m.numel() // n if n else 0
     idx = torch.empty(m.shape, dtype=torch.int32, device=m.device)
     cnt = torch.empty(m.shape[:-1], dtype=torch.int32, device=m.device)
-    with torch.cuda.device(m.device):
+    with _on_device(m):
         st = _lib.load().lvar_mask_to_lists(m.data_ptr(), n, idx.data_ptr(), n, cnt.data_ptr(), rows, n,
                                            int(multiple_of), _stream(m))
     _lib.check(st, "lvar_mask_to_lists")
