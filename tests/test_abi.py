@@ -60,6 +60,41 @@ def test_argument_validation_without_device(lib):
     assert lib.lvar_block_sparse_attn_fwd(fake, fake, fake, fake, None, None, None, 0, 0, one, 0, 0, 4, 4, 128, 64, 1, 1, 16, 16, 128, 1.0, None) == -1
 
 
+def test_list_build_and_upsample_argument_validation(lib):
+    from lvar_amd._lib import LvarTensor
+    null = LvarTensor(None, 0, 0, 0)
+    fake = LvarTensor(0x1000, 128 * 16 * 128, 16 * 128, 128)
+    one = ctypes.c_void_p(0x2000)
+    assert lib.lvar_topk_token_lists(None, 100, one, 100, one, 4, 100, 10, None) == -1            # no scores
+    assert lib.lvar_topk_token_lists(one, 100, one, 100, one, 4, 100, 101, None) == -1            # k > Lk
+    assert lib.lvar_topk_token_lists(one, 99, one, 100, one, 4, 100, 10, None) == -1              # row stride < Lk
+    assert lib.lvar_topk_token_lists(one, 100, one, 5, one, 4, 100, 10, None) == -1               # output row shorter than k
+    assert lib.lvar_topk_token_lists(one, 100, one, 100, one, 0, 100, 10, None) == 0              # no rows: nothing to launch
+    assert lib.lvar_remap_concat_lists(one, 100, 100, None, 0, 8, one, 200, one, 2, 3, 4, 64, 500, None) == -1   # local run without a table
+    assert lib.lvar_remap_concat_lists(one, 100, 100, one, 8, 8, one, 70, one, 2, 3, 4, 64, 500, None) == -1     # 64 + 8 > output row
+    assert lib.lvar_remap_concat_lists(one, 100, 100, None, 0, 0, one, 64, one, 2, 0, 4, 64, 500, None) == -1    # no source groups
+    assert lib.lvar_mask_to_lists(one, 10, one, 10, one, 3, 10, 0, None) == -1                    # multiple_of must be positive
+    assert lib.lvar_mask_to_lists(one, 10, one, 9, one, 3, 10, 1, None) == -1                     # output row shorter than n
+    assert lib.lvar_mask_to_lists(one, 10, one, 10, one, 0, 10, 1, None) == 0
+    # fused upsample: Lq must be dst_side^2 and the cache must exist
+    args = (one, one, 1, 16, 192, 1, 1, 16, 16, 128, 1.0, 1.0, None)
+    assert lib.lvar_csp_attn_upsample_fwd(fake, fake, fake, fake, 2, 5, fake, None, None, *args) == -1         # 25 != 16
+    assert lib.lvar_csp_attn_upsample_fwd(fake, fake, fake, null, 2, 4, fake, None, None, *args) == -1
+
+
+def test_header_is_plain_c(tmp_path):
+    """The public header must be usable from C (the reference's other bindings are C/C++)."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "use.c"
+    src.write_text('#include "lvar_sparse_attn.h"\nint main(void) { lvar_tensor_t t = {0, 0, 0, 0}; (void)t; return lvar_version() ? 0 : 1; }\n')
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.dirname(HEADER), "-c", str(src),
+                        "-o", str(tmp_path / "use.o")], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
 def test_python_wrappers_fail_loudly_without_gpu():
     import torch
     from lvar_amd import sparse_attn_ops as ops
