@@ -187,6 +187,22 @@ int lvar_mask_to_lists(const uint8_t* mask, int64_t mask_row_stride,
                        int32_t* indices, int64_t idx_row_stride, int32_t* counts,
                        int rows, int n, int multiple_of, void* stream);
 
+/*
+ * Window-query key scores: for every (batch, head)
+ *   s[n]      = scale * sum_{i < n_window} q[row(window_keys[i])] . k[n],   row(x) = clamp(x - (Lk - Lq), 0, Lq-1),
+ *   s[n]      = -inf at the window's own keys n in window_keys,
+ *   scores[n] = pool_{|m - n| <= pool_kernel_size/2} s[m]   (average with zero padding, or maximum),
+ *   scores[n] = -inf again at the window's own keys.
+ * q [B,H,Lq,d] holds the queries of the newest Lq of the Lk keys; window_keys is int64 [B,H,n_window]
+ * (key positions, repeats count twice), scores fp32 contiguous [B,H,Lk]; pool_kernel_size odd, <= 33.
+ * One pass over K with the summed window query (fp32).  Replaces the query gather, the
+ * [n_window x Lk] matmul, masking, sum and pooling of ScaleKV's cache selection
+ * (models/scalekv/scale_kv.py:233-262), which rounds every logit to bf16 before summing.
+ */
+int lvar_window_key_scores(lvar_tensor_t q, lvar_tensor_t k, const int64_t* window_keys, int n_window,
+                           float* scores, int B, int H, int Lq, int Lk, int head_dim,
+                           int pool_kernel_size, int max_pool, float scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

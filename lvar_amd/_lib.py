@@ -15,6 +15,7 @@ EXPORTED_SYMBOLS = (
     "lvar_dense_attn_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_csp_attn_upsample_fwd",
     "lvar_block_sparse_attn_fwd",
     "lvar_block_topk_lists", "lvar_topk_token_lists", "lvar_remap_concat_lists", "lvar_mask_to_lists",
+    "lvar_window_key_scores",
 )
 
 
@@ -66,6 +67,8 @@ def load() -> C.CDLL:
     lib.lvar_remap_concat_lists.argtypes = [P, I64, I, P, I64, I, P, I64, P, I, I, I, I, I, P]
     lib.lvar_mask_to_lists.restype = I
     lib.lvar_mask_to_lists.argtypes = [P, I64, P, I64, P, I, I, I, P]
+    lib.lvar_window_key_scores.restype = I
+    lib.lvar_window_key_scores.argtypes = [T, T, P, I, P, I, I, I, I, I, I, I, F, P]
     _lib = lib
     return lib
 

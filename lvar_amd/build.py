@@ -17,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "liblvar_sparse_attn.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["attn_fwd.hip", "colsum.hip", "masklist.hip", "listbuild.hip", "capi.hip"]
+SOURCES = ["attn_fwd.hip", "colsum.hip", "masklist.hip", "listbuild.hip", "windowscore.hip", "capi.hip"]
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off: hipcc must not form v_pk_{add,mul,fma}_f32 from float code
 # -fno-honor-nans -mno-amdgpu-ieee: max/min map to single v_max/v_max3 without NaN-quieting copies

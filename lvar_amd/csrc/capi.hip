@@ -214,4 +214,19 @@ int lvar_mask_to_lists(const uint8_t* mask, int64_t mask_row_stride, int32_t* in
   return launch_mask_to_lists(p, (hipStream_t)stream);
 }
 
+int lvar_window_key_scores(lvar_tensor_t q, lvar_tensor_t k, const int64_t* window_keys, int n_window,
+                           float* scores, int B, int H, int Lq, int Lk, int head_dim,
+                           int pool_kernel_size, int max_pool, float scale, void* stream) {
+  if (!view_ok(q) || !view_ok(k) || !scores || B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || Lq > Lk || n_window < 0 ||
+      (n_window > 0 && !window_keys) || !std::isfinite(scale))
+    return LVAR_EINVAL;
+  WinScoreParams p{};
+  p.q = (const bf16_t*)q.ptr; p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sr = q.stride_row;
+  p.k = (const bf16_t*)k.ptr; p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sr = k.stride_row;
+  p.window = window_keys; p.out = scores;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk; p.W = n_window; p.ksize = pool_kernel_size; p.maxpool = max_pool ? 1 : 0;
+  p.scale = scale;
+  return launch_window_scores(p, head_dim, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -94,6 +94,16 @@ inline bool ensure_lds_limit(const void* kernel, int bytes, std::atomic<uint64_t
   return true;
 }
 
+struct WinScoreParams {
+  const bf16_t *q, *k;
+  const int64_t* window;  // [B*H, W] key positions of the window tokens
+  float* out;             // [B*H, Lk]
+  int64_t q_sb, q_sh, q_sr, k_sb, k_sh, k_sr;
+  int B, H, Lq, Lk, W, ksize, maxpool, nchunks;
+  float scale;
+};
+
+int launch_window_scores(const WinScoreParams& p, int head_dim, hipStream_t s);
 int launch_topk_token_lists(const TopkListParams& p, hipStream_t s);
 int launch_remap_concat_lists(const RemapListParams& p, hipStream_t s);
 int launch_mask_to_lists(const MaskCompactParams& p, hipStream_t s);

@@ -1,0 +1,89 @@
+// Window-query key scores (the scoring step of a ScaleKV-style cache selection): the logits of a small
+// set of "window" queries against every key are summed over the queries, smoothed by a 1-D pool
+// along the key axis and masked at the window's own keys.  Since sum_i (q_i . k_n) = (sum_i q_i) . k_n
+// the work is one pass over K with a single summed query: HBM-bound (2 bytes x d per key), no MFMA.
+#include "common.h"
+#include "launch.h"
+
+namespace lvar {
+
+constexpr int WS_KEYS = 256;   // keys per workgroup
+constexpr int WS_MAXR = 16;    // largest pool radius (kernel_size <= 33)
+
+template <int D>
+__global__ __launch_bounds__(256) void window_scores_kernel(const WinScoreParams p) {
+  constexpr int LPR = D / 8;          // lanes that share one key row (8 bf16 = 16 bytes each)
+  constexpr int RPP = 256 / LPR;      // key rows per pass of the workgroup
+  __shared__ float qs[D];
+  __shared__ float sc[WS_KEYS + 2 * WS_MAXR];
+  __shared__ uint8_t wm[WS_KEYS + 2 * WS_MAXR];
+  const int tid = threadIdx.x;
+  const int bh = blockIdx.x / p.nchunks, chunk = blockIdx.x - bh * p.nchunks;
+  const int b = bh / p.H, h = bh - b * p.H;
+  const int r = p.ksize >> 1;
+  const int n0 = chunk * WS_KEYS - r;  // key of sc[0]
+  const int span = WS_KEYS + 2 * r;
+  const int64_t* win = p.window + (int64_t)bh * p.W;
+  const bf16_t* qb = p.q + b * p.q_sb + h * p.q_sh;
+  const bf16_t* kb = p.k + b * p.k_sb + h * p.k_sh;
+
+  // summed window query, fp32; a window key n is the query row clamp(n - (Lk - Lq), 0, Lq-1)
+  for (int c = tid; c < D; c += 256) {
+    float acc = 0.f;
+    for (int i = 0; i < p.W; i++) {
+      const int row = max(0, min(p.Lq - 1, (int)win[i] - (p.Lk - p.Lq)));
+      acc += (float)qb[(int64_t)row * p.q_sr + c];
+    }
+    qs[c] = acc;
+  }
+  __syncthreads();
+
+  const int g = tid / LPR, l = tid - g * LPR;
+  float qv[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) qv[e] = qs[l * 8 + e];
+  const float pad = p.maxpool ? -INFINITY : 0.f;
+  for (int j = g; j < span; j += RPP) {
+    const int n = n0 + j;
+    float dot = 0.f;
+    if (n >= 0 && n < p.Lk) {
+      const u32x4 kv = *(const u32x4*)(kb + (int64_t)n * p.k_sr + l * 8);
+#pragma unroll
+      for (int e = 0; e < 4; e++) dot += bf16_lo(kv[e]) * qv[2 * e] + bf16_hi(kv[e]) * qv[2 * e + 1];
+    }
+#pragma unroll
+    for (int m = LPR >> 1; m > 0; m >>= 1) dot += __shfl_xor(dot, m, 64);
+    if (l == 0) {
+      sc[j] = (n >= 0 && n < p.Lk) ? dot * p.scale : pad;
+      wm[j] = 0;
+    }
+  }
+  __syncthreads();
+  // the window's own keys do not compete: -inf before the pool (it spreads to their neighbours under
+  // an average) and again after it
+  for (int i = tid; i < p.W; i += 256) {
+    const int j = (int)win[i] - n0;
+    if (j >= 0 && j < span) { sc[j] = -INFINITY; wm[j] = 1; }
+  }
+  __syncthreads();
+  const int n = chunk * WS_KEYS + tid;
+  if (n < p.Lk) {
+    float acc = p.maxpool ? -INFINITY : 0.f;
+    for (int e = 0; e <= 2 * r; e++) acc = p.maxpool ? fmaxf(acc, sc[tid + e]) : acc + sc[tid + e];
+    if (!p.maxpool) acc = acc / (float)p.ksize;
+    p.out[(int64_t)bh * p.Lk + n] = wm[tid + r] ? -INFINITY : acc;
+  }
+}
+
+int launch_window_scores(const WinScoreParams& p0, int head_dim, hipStream_t stream) {
+  WinScoreParams p = p0;
+  if ((p.ksize & 1) == 0 || p.ksize < 1 || (p.ksize >> 1) > WS_MAXR) return LVAR_EUNSUPPORTED;
+  p.nchunks = (p.Lk + WS_KEYS - 1) / WS_KEYS;
+  const dim3 grid(p.B * p.H * p.nchunks);
+  if (head_dim == 128) hipLaunchKernelGGL(window_scores_kernel<128>, grid, dim3(256), 0, stream, p);
+  else if (head_dim == 64) hipLaunchKernelGGL(window_scores_kernel<64>, grid, dim3(256), 0, stream, p);
+  else return LVAR_EUNSUPPORTED;
+  return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
+}
+
+}  // namespace lvar

@@ -423,3 +423,43 @@ def mask_to_lists(mask, multiple_of: int = 1):
                                            int(multiple_of), _stream(m))
     _lib.check(st, "lvar_mask_to_lists")
     return cnt, idx
+
+
+def window_key_scores(q, k, window_keys, kernel_size: int = 5, pooling: str = "avgpool", scale=None):
+    """Scores of all keys against a small set of window queries, as ScaleKV's cache selection computes them
+    (models/scalekv/scale_kv.py:233-262): the logits of the window's queries are summed per key (scaled by
+    ``1/sqrt(d)`` unless ``scale`` is given), the window's own keys are set to ``-inf``, the result is pooled
+    along the key axis (``avgpool`` with zero padding or ``maxpool``, odd ``kernel_size``, stride 1) and masked
+    again.  ``q`` ``[B,H,Lq,d]`` are the queries of the newest ``Lq`` keys of ``k`` ``[B,H,Lk,d]``;
+    ``window_keys`` int64 ``[B,H,W]`` are key positions.  Returns fp32 ``[B,H,Lk]``.  One pass over K."""
+    q, k = _prep(q, "q"), _prep(k, "k")
+    _check_qkv(q, k, k)
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    _require(Lq <= Lk, "q holds the queries of the newest keys: Lq must not exceed Lk")
+    _require(pooling in ("avgpool", "maxpool"), "pooling must be 'avgpool' or 'maxpool'")
+    _require(kernel_size % 2 == 1 and 1 <= kernel_size <= 33, "kernel_size must be odd and at most 33")
+    _require(window_keys.dim() == 3 and tuple(window_keys.shape[:2]) == (B, H), "window_keys must be [B,H,W]")
+    win = window_keys.to(device=q.device, dtype=torch.int64).contiguous()
+    out = torch.empty((B, H, Lk), dtype=torch.float32, device=q.device)
+    with _on_device(q):
+        st = _lib.load().lvar_window_key_scores(_view(q), _view(k), win.data_ptr(), win.shape[2], out.data_ptr(),
+                                               B, H, Lq, Lk, d, int(kernel_size), 1 if pooling == "maxpool" else 0,
+                                               _scale(q, scale), _stream(q))
+    _lib.check(st, "lvar_window_key_scores")
+    return out
+
+
+def scalekv_keep_indices(q, k, window_keys, max_capacity: int, kernel_size: int = 5, pooling: str = "avgpool"):
+    """Key positions a ScaleKV-style cache keeps (models/scalekv/scale_kv.py:229-282): the window keys plus
+    the ``max_capacity - W`` best-scoring other keys, ascending; int64 ``[B,H,min(max_capacity, Lk)]``.
+    Scores and the top-k selection run in the HIP library (ties go to the smaller key position)."""
+    B, H, W = window_keys.shape
+    Lk = k.shape[2]
+    keep = min(max(0, int(max_capacity) - W), Lk - W)
+    if keep <= 0:
+        return torch.sort(window_keys.to(torch.int64), dim=-1).values
+    scores = window_key_scores(q, k, window_keys, kernel_size, pooling)
+    rest, _ = topk_token_lists(scores, keep, out_len=keep)
+    combined = torch.cat([rest.to(torch.int64), window_keys.to(device=rest.device, dtype=torch.int64)], dim=-1)
+    return torch.sort(combined, dim=-1).values

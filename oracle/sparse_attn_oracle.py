@@ -28,7 +28,7 @@ __all__ = [
     "map_inds_counts_across_scales", "local_window_indices", "crossscale_self_indices",
     "aggregate_group_indices", "upsample_ocache", "flex_block_mask", "infinity_cum",
     "INFINITY_SCALES", "config2_block_mask", "attn_flops_blocks", "attn_flops_lists",
-    "topk_token_set", "append_local_run", "mask_to_lists",
+    "topk_token_set", "append_local_run", "mask_to_lists", "window_key_scores",
 ]
 
 # Infinity "1M" scale schedule, reference utils/dynamic_resolution.py:7 and
@@ -308,6 +308,30 @@ def mask_to_lists(mask, multiple_of=1):
         idx[r, :len(row)] = row
         cnt[r] = len(row)
     return torch.from_numpy(cnt.reshape(m.shape[:-1])), torch.from_numpy(idx.reshape(m.shape))
+
+
+def window_key_scores(q, k, window_keys, kernel_size=5, pooling="avgpool", dtype=torch.float32):
+    """Masked, pooled key scores of ScaleKV's cache selection, models/scalekv/scale_kv.py:233-262: gather
+    the window's queries (``local = clamp(window - (Lk - Lq), 0, Lq-1)``), logits against all keys divided
+    by sqrt(d), ``-inf`` at the window's own keys, sum over the window queries, 1-D pool along the keys
+    (padding ``kernel_size//2``, stride 1), ``-inf`` at the window keys again.  The reference does this
+    in bf16 tensors; here in ``dtype``.  Returns [B,H,Lk]."""
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    local = torch.clamp(window_keys - (Lk - Lq), 0, Lq - 1)
+    wq = torch.gather(q.to(dtype), 2, local.unsqueeze(-1).expand(-1, -1, -1, d))
+    w = torch.matmul(wq, k.to(dtype).transpose(2, 3)) / math.sqrt(d)
+    mask = torch.ones(B, H, 1, Lk, dtype=torch.bool)
+    mask.scatter_(3, window_keys.unsqueeze(2), False)
+    w = w.masked_fill(~mask, float("-inf"))
+    s = w.sum(dim=2)
+    if pooling == "avgpool":
+        pooled = torch.nn.functional.avg_pool1d(s, kernel_size, padding=kernel_size // 2, stride=1)
+    else:
+        pooled = torch.nn.functional.max_pool1d(s, kernel_size, padding=kernel_size // 2, stride=1)
+    pooled = pooled.clone()
+    pooled.scatter_(2, window_keys, float("-inf"))
+    return pooled
 
 
 def local_window_indices(Hh, W, base, win):

@@ -239,3 +239,34 @@ def test_ops_replay_correctly_from_a_hip_graph():
         torch.cuda.synchronize()
         for a, b in zip(outs, eager):
             assert torch.equal(a, b), rep
+
+
+@pytest.mark.gpu
+def test_window_key_scores_and_scalekv_selection():
+    import oracle
+    from lvar_amd import sparse_attn_ops as ops
+    g = torch.Generator().manual_seed(15)
+    for (B, H, Lq, Lk, d, W, ks, pooling) in ((1, 2, 400, 921, 128, 16, 5, "avgpool"), (2, 3, 64, 700, 64, 9, 7, "maxpool"),
+                                              (1, 1, 300, 300, 128, 4, 1, "avgpool"), (1, 2, 1024, 2521, 128, 256, 5, "maxpool")):
+        q = (torch.randn(B, H, Lq, d, generator=g) * 0.5).to(torch.bfloat16)
+        k = (torch.randn(B, H, Lk, d, generator=g) * 0.5).to(torch.bfloat16)
+        win = torch.randint(Lk - Lq, Lk, (B, H, W), generator=g)
+        if W >= 9:
+            win[..., 1] = win[..., 0]                                     # a repeated window token
+            win[..., 2] = Lk - 1                                          # the last key: pooling at the border
+        got = ops.window_key_scores(q.cuda(), k.cuda(), win.cuda(), ks, pooling).cpu()
+        ref = oracle.window_key_scores(q, k, win, ks, pooling)
+        inf = torch.isinf(ref)
+        assert torch.equal(torch.isinf(got), inf), (Lq, Lk, pooling)
+        assert torch.allclose(got[~inf], ref[~inf], rtol=1e-3, atol=1e-3)
+        keep = ops.scalekv_keep_indices(q.cuda(), k.cuda(), win.cuda(), W + 50, ks, pooling).cpu()
+        assert keep.shape == (B, H, W + 50) and bool((keep[..., 1:] >= keep[..., :-1]).all())
+        # the kept non-window keys are a top-50 set of the library's own scores
+        sc = got.clone()
+        for b in range(B):
+            for h in range(H):
+                rest = [x for x in keep[b, h].tolist() if x not in set(win[b, h].tolist())]
+                if torch.isinf(sc[b, h]).sum() <= Lk - 50:
+                    assert len(rest) == 50
+                    thr = torch.topk(sc[b, h], 50).values[-1]
+                    assert bool((sc[b, h, rest] >= thr).all())

@@ -294,3 +294,26 @@ def test_append_local_run_layout():
     out, counts = oracle.append_local_run(inds, 4, local, 2, 9)
     assert out.shape == (2, 1, 3, 9) and counts.tolist() == [[[6] * 3]] * 2
     assert out[1, 0, 2].tolist() == [50, 51, 52, 53, 300, 301, 0, 0, 0]
+
+
+def test_window_key_scores_bruteforce():
+    """Pure-Python restatement of the masked, summed, pooled window logits on a tiny case."""
+    B, H, Lq, Lk, d, ks = 1, 2, 6, 11, 4, 3
+    q, k = rnd(B, H, Lq, d, seed=31), rnd(B, H, Lk, d, seed=32)
+    win = torch.tensor([[[5, 7, 10], [6, 6, 9]]])                       # key positions; a repeat in head 1
+    for pooling in ("avgpool", "maxpool"):
+        got = oracle.window_key_scores(q, k, win, ks, pooling, dtype=torch.float64)
+        for h in range(H):
+            wk = win[0, h].tolist()
+            raw = []
+            for n in range(Lk):
+                if n in wk:
+                    raw.append(-math.inf)
+                else:
+                    raw.append(sum(sum(float(q[0, h, min(max(x - (Lk - Lq), 0), Lq - 1), c]) * float(k[0, h, n, c]) for c in range(d))
+                                   for x in wk) / math.sqrt(d))
+            for n in range(Lk):
+                nb = [raw[m] if 0 <= m < Lk else (0.0 if pooling == "avgpool" else -math.inf) for m in range(n - 1, n + 2)]
+                exp = -math.inf if n in wk else (sum(nb) / ks if pooling == "avgpool" else max(nb))
+                g = float(got[0, h, n])
+                assert (g == exp) if math.isinf(exp) else abs(g - exp) < 1e-9, (pooling, h, n, g, exp)
