@@ -15,6 +15,7 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const WinScoreParams
   constexpr int LPR = D / 8;          // lanes that share one key row (8 bf16 = 16 bytes each)
   constexpr int RPP = 256 / LPR;      // key rows per pass of the workgroup
   __shared__ float qs[D];
+  __shared__ float part[RPP][D];
   __shared__ float sc[WS_KEYS + 2 * WS_MAXR];
   __shared__ uint8_t wm[WS_KEYS + 2 * WS_MAXR];
   const int tid = threadIdx.x;
@@ -27,18 +28,29 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const WinScoreParams
   const bf16_t* qb = p.q + b * p.q_sb + h * p.q_sh;
   const bf16_t* kb = p.k + b * p.k_sb + h * p.k_sh;
 
-  // summed window query, fp32; a window key n is the query row clamp(n - (Lk - Lq), 0, Lq-1)
+  // summed window query, fp32; a window key n is the query row clamp(n - (Lk - Lq), 0, Lq-1).
+  // Row group g (LPR lanes, 16 bytes each) adds up the window rows g, g + RPP, ...; the RPP partial
+  // sums meet in LDS.
+  const int g = tid / LPR, l = tid - g * LPR;
+  {
+    float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int i = g; i < p.W; i += RPP) {
+      const int row = max(0, min(p.Lq - 1, (int)win[i] - (p.Lk - p.Lq)));
+      const u32x4 qv4 = *(const u32x4*)(qb + (int64_t)row * p.q_sr + l * 8);
+#pragma unroll
+      for (int e = 0; e < 4; e++) { a[2 * e] += bf16_lo(qv4[e]); a[2 * e + 1] += bf16_hi(qv4[e]); }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) part[g][l * 8 + e] = a[e];
+  }
+  __syncthreads();
   for (int c = tid; c < D; c += 256) {
     float acc = 0.f;
-    for (int i = 0; i < p.W; i++) {
-      const int row = max(0, min(p.Lq - 1, (int)win[i] - (p.Lk - p.Lq)));
-      acc += (float)qb[(int64_t)row * p.q_sr + c];
-    }
+    for (int gg = 0; gg < RPP; gg++) acc += part[gg][c];
     qs[c] = acc;
   }
   __syncthreads();
 
-  const int g = tid / LPR, l = tid - g * LPR;
   float qv[8];
 #pragma unroll
   for (int e = 0; e < 8; e++) qv[e] = qs[l * 8 + e];
