@@ -73,6 +73,31 @@ def main():
     csla = oracle.flex_block_mask(8, [-1, -1, -1, -1, 1, 1, 3, 5, 7], 3, 128)
     np.savez_compressed(os.path.join(HERE, "list_build_constants.npz"), runs11=runs11.numpy(), runs12=runs12.numpy(),
                         csla_scale8=csla.numpy(), cum=np.array(oracle.infinity_cum(), dtype=np.int64))
+    # 5. list kernels of the sparse step: token top-k set (with ties through the cut), group remap + local run,
+    #    mask compaction with count padding, O-cache upsample + column-sparse attention, window-query key scores
+    sc = torch.rand(2, 3, 700, generator=g)
+    sc[0, 0, ::2] = 0.5
+    topk = oracle.topk_token_set(sc, 128)
+    src = torch.randint(0, 1000, (1, 2, 9, 300), generator=g, dtype=torch.int32)
+    local = torch.randint(0, 900, (12, 64), generator=g)
+    rm, rc = oracle.map_inds_counts_across_scales(src, torch.full((1, 2, 9), 192, dtype=torch.int32), 2304, 900)
+    rl, rlc = oracle.append_local_run(rm, 192, local, 64, 900)
+    msk = torch.rand(3, 4, 165, generator=g) < 0.2
+    mc, mi = oracle.mask_to_lists(msk, 64)
+    q, k, v = qkv(1, 2, 64, 200, 128, seed=105, amp=0.5)
+    cache = torch.randn(1, 2, 25, 128, generator=g).to(torch.bfloat16)
+    uidx = torch.zeros(1, 2, 1, 200, dtype=torch.int32)
+    for h in range(2):
+        uidx[0, h, 0, :64] = torch.randperm(200, generator=g)[:64].to(torch.int32)
+    ucnt = torch.full((1, 2, 1), 64, dtype=torch.int32)
+    up = oracle.csp_attn(q, k, v, None, uidx, ucnt, oracle.upsample_ocache(cache, 25, 64), 1, dtype=torch.float64)
+    win = torch.randint(136, 200, (1, 2, 9), generator=g)
+    ws = oracle.window_key_scores(q, k, win, 5, "avgpool", dtype=torch.float64)
+    np.savez_compressed(os.path.join(HERE, "list_kernels.npz"), scores=f32(sc), topk128=topk.numpy(), src=src.numpy(), local=local.numpy(),
+                        remap_concat=rl.numpy(), remap_counts=rlc.numpy(), mask=msk.numpy(), mask_counts=mc.numpy(), mask_idx=mi.numpy(),
+                        q=bits(q), k=bits(k), v=bits(v), cache=bits(cache), uidx=uidx.numpy(), ucnt=ucnt.numpy(), upsampled_out=f32(up),
+                        window=win.numpy(), window_scores=f32(ws))
+
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)) // 1024, "KiB")

@@ -104,3 +104,39 @@ def test_hip_matches_sparse_fixtures():
                                       t(z["num"]).cuda(), t(z["idx"]).cuda(), 128, 64)
     assert close(o.float().cpu(), t(z["o"]), 2e-2, 1e-2)
     assert close((M + torch.log2(L)).cpu(), t(z["lse2"]), 1e-3, 0)
+
+
+def test_oracle_and_host_mirrors_reproduce_list_kernel_fixture():
+    from lvar_amd import mask_build as mb
+    z = load("list_kernels.npz")
+    assert torch.equal(oracle.topk_token_set(t(z["scores"]), 128), t(z["topk128"]))
+    # the torch host mirrors (CPU path of lvar_amd.mask_build) give the same lists
+    inds, counts = mb.topk_index_list(t(z["scores"]).unsqueeze(0), 128 / 700, multiple_of=64, order="index")
+    assert int(counts[0, 0, 0]) == 128 and torch.equal(inds[0, ..., :128], t(z["topk128"]))
+    a, c = mb.map_inds_counts_across_scales(t(z["src"]), 192, 2304, 900)
+    out, cnt = mb.append_local_run(a, 192, t(z["local"]), 64, 900, multiple_of=64)
+    assert torch.equal(out, t(z["remap_concat"])) and torch.equal(cnt, t(z["remap_counts"]))
+    mc, mi = oracle.mask_to_lists(t(z["mask"]), 64)
+    assert torch.equal(mc, t(z["mask_counts"])) and torch.equal(mi, t(z["mask_idx"]))
+    ws = oracle.window_key_scores(bf16(z["q"]), bf16(z["k"]), t(z["window"]), 5, "avgpool", dtype=torch.float64)
+    ref = t(z["window_scores"])
+    assert torch.equal(torch.isinf(ws), torch.isinf(ref)) and close(ws[~torch.isinf(ref)].float(), ref[~torch.isinf(ref)], 1e-5, 1e-5)
+
+
+@pytest.mark.gpu
+def test_hip_matches_list_kernel_fixture():
+    from lvar_amd import sparse_attn_ops as ops
+    z = load("list_kernels.npz")
+    idx, cnt = ops.topk_token_lists(t(z["scores"]).cuda(), 128)
+    assert torch.equal(idx[..., :128].cpu(), t(z["topk128"])) and bool((cnt == 128).all())
+    out, counts = ops.remap_concat_lists(t(z["src"]).cuda(), 192, 2304, 900, t(z["local"]).cuda())
+    assert torch.equal(out.cpu(), t(z["remap_concat"])) and torch.equal(counts.cpu(), t(z["remap_counts"]))
+    mc, mi = ops.mask_to_lists(t(z["mask"]).cuda(), 64)
+    assert torch.equal(mc.cpu(), t(z["mask_counts"])) and torch.equal(mi.cpu(), t(z["mask_idx"]))
+    q, k, v, cache = (bf16(z[n]).cuda() for n in ("q", "k", "v", "cache"))
+    up = ops.csp_attn_upsampled(q, k, v, None, t(z["uidx"]).cuda(), t(z["ucnt"]).cuda(), cache, 1)
+    assert close(up.float().cpu(), t(z["upsampled_out"]), 2e-2, 1e-2)
+    ws = ops.window_key_scores(q, k, t(z["window"]).cuda(), 5, "avgpool").cpu()
+    ref = t(z["window_scores"])
+    fin = ~torch.isinf(ref)
+    assert torch.equal(torch.isinf(ws), ~fin) and close(ws[fin], ref[fin], 1e-3, 1e-3)
