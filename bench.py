@@ -309,7 +309,7 @@ def main():
     SETTLE_MS = args.settle_ms
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the hot path on ONE GPU; --gpus N with N > 1 is not supported "
-              "(the path shards over (batch, head) with no exchange step, see DESIGN.md).", file=sys.stderr)
+              "(the path shards over (batch, head) with no exchange step: give every GPU its own heads).", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (no CPU fallback)", file=sys.stderr)
