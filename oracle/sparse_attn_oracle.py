@@ -107,7 +107,7 @@ def colsum_from_lse(q, k, M, L, scale=None, q_group_size=192, dtype=torch.float3
 
 def key_block_sums(cs, block_k=64):
     """Sum of colsum over blocks of ``block_k`` consecutive keys, ragged last block.
-    Not in the reference (it ranks key tokens); defined by BASELINE config 1/3."""
+    Not in the reference (it ranks key tokens); defined by the benchmark configurations (per-64-key block sums of the colsum)."""
     Lk = cs.shape[-1]
     nb = (Lk + block_k - 1) // block_k
     pad = nb * block_k - Lk
@@ -449,7 +449,7 @@ def flex_block_mask(q_scale_idx, kernel_schedule, attn_sink_scale, block_size=12
 
 def config2_block_mask(colsum_blocks, block_q=128, block_k=64, density=0.25, sink_scale=7, window=2,
                        scales=INFINITY_SCALES):
-    """BASELINE config 2 mask for the last Infinity scale: key blocks of scales < ``sink_scale``
+    """Headline-benchmark mask for the last Infinity scale: key blocks of scales < ``sink_scale``
     (kv < cum[7] = 521) always kept, plus +-``window`` key blocks around the query block's
     rescaled position in every later scale, plus the top-ranked remainder by ``colsum_blocks``
     [B,H,nQ,nK] until ``round(density*nK)`` blocks per row.  Returns bool [B,H,nQ,nK]."""

@@ -34,7 +34,7 @@ def f32(t):
 
 
 def main():
-    # 1. VAR-d16 last scale (BASELINE config 1), one batch x two heads: dense + colsum + block sums + top-5 blocks
+    # 1. VAR-d16 last scale (the CPU-runnable benchmark case), one batch x two heads: dense + colsum + block sums + top-5 blocks
     q, k, v = qkv(1, 1, 256, 680, 64, seed=101)
     o, cs, (M, L) = oracle.dense_colsum_attn(q, k, v, dtype=torch.float64)
     _, cs_all, _ = oracle.dense_colsum_attn(q, k, v, q_group_size=256, dtype=torch.float64)

@@ -36,7 +36,7 @@ def test_oracle_reproduces_var_d16_fixture():
     assert close(M + torch.log2(L), t(z["lse2"]), 1e-4, 0)
     bs = oracle.key_block_sums(t(z["cs_all"]), 64)
     assert close(bs, t(z["block_sums"]), 1e-5, 1e-5) and bs.shape[-1] == 11
-    # BASELINE config 1: keep 64*round(0.5*680/64)/64 = 5 of 11 key blocks; mask is exact given the colsum
+    # VAR-d16 benchmark case: keep 64*round(0.5*680/64)/64 = 5 of 11 key blocks; mask is exact given the colsum
     top = torch.topk(t(z["block_sums"]), k=oracle.indices_count(0.5, 680, 64) // 64, dim=-1).indices.sort(-1).values
     assert torch.equal(top.to(torch.int32), t(z["top5_blocks"]))
 

@@ -36,7 +36,7 @@ def check_lse(M_gpu, L_gpu, M_ref, L_ref):
 
 
 DENSE_SHAPES = [
-    (2, 16, 256, 680, 64),    # VAR-d16 last scale (BASELINE config 1 shape)
+    (2, 16, 256, 680, 64),    # VAR-d16 last scale (the CPU-runnable benchmark shape)
     (1, 2, 300, 1000, 128),   # ragged Lq and Lk
     (1, 3, 128, 64, 128),     # exactly one key tile
     (1, 2, 33, 25, 128),      # fewer keys than one tile, Lq not a multiple of 32

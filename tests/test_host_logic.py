@@ -107,7 +107,7 @@ def test_block_lists_and_sums_match_oracle():
     cs = torch.rand(1, 2, 3, 680, generator=torch.Generator().manual_seed(4))
     assert torch.allclose(mb.key_block_sums(cs, 64), oracle.key_block_sums(cs, 64))
     num, idx = mb.topk_block_lists(mb.key_block_sums(cs, 64), 0.5, k_len=680)
-    assert int(num[0, 0, 0]) == 5                              # 64*round(0.5*680/64)/64, BASELINE config 1
+    assert int(num[0, 0, 0]) == 5                              # 64*round(0.5*680/64)/64, VAR-d16 benchmark case
     assert int(mb.topk_block_lists(mb.key_block_sums(cs, 64), 0.5)[0][0, 0, 0]) == 6   # round(5.5), half-to-even
     assert bool((idx[..., 1:] > idx[..., :-1]).all())
 

@@ -1,7 +1,7 @@
 """Pins the CPU oracle (oracle/sparse_attn_oracle.py) against things it does not itself define:
 library routines (SDPA, logsumexp, F.interpolate, torch.sort), brute-force pure-Python loops on tiny
 inputs, closed-form special cases and the known answers written in the reference's sources
-(models/sparvar/sparse_attn.py:909,913,934; BASELINE config 1).  The reference ships no golden
+(models/sparvar/sparse_attn.py:909,913,934; the VAR-d16 benchmark case).  The reference ships no golden
 vectors for this path, so these checks are what anchors parity."""
 import math
 
@@ -78,7 +78,7 @@ def test_indices_count_known_answers():
     # decision scale of Infinity-2B: Lk = 4121, top_keys = 0.2 (sparse-attn-config.yml:20)
     assert oracle.indices_count(0.2, 4121, 64) == 832
     assert oracle.indices_count(0.2, 4121, 112) == 784
-    # BASELINE config 1: Lk = 680, keep 50 % => 320 tokens = 5 blocks of 64
+    # VAR-d16 benchmark case: Lk = 680, keep 50 % => 320 tokens = 5 blocks of 64
     assert oracle.indices_count(0.5, 680, 64) == 320
     # half-to-even: 0.25*640/64 = 2.5 -> 2
     assert oracle.indices_count(0.25, 640, 64) == 128
