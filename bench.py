@@ -64,6 +64,27 @@ def block_flops(num, idx, Lq, Lk, d, bq, bk, B, H):
 SETTLE_MS = 150.0   # untimed load before the warm-up steps; set from --settle-ms
 
 
+def device_summary():
+    """Name, CU count and maximum engine clock of the GPU as `rocminfo` reports them, and the bf16 MFMA
+    rate they imply (4096 flop per clock per CU: four SIMDs, one 32x32x16 MFMA = 32768 flop in 32 cycles
+    each).  The roofline peak stays the published figure; this line shows what the part in hand can do."""
+    import re
+    import subprocess
+    pr = torch.cuda.get_device_properties(0)
+    out = {"name": pr.name, "arch": pr.gcnArchName, "cus": pr.multi_processor_count, "hbm_gib": round(pr.total_memory / 2 ** 30, 1)}
+    try:
+        txt = subprocess.run(["/opt/rocm/bin/rocminfo"], capture_output=True, text=True, timeout=30).stdout
+        for agent in txt.split("*******")[1:]:
+            if re.search(r"Name:\s+gfx950", agent):
+                mhz = int(re.search(r"Max Clock Freq\. \(MHz\):\s+(\d+)", agent).group(1))
+                cus = int(re.search(r"Compute Unit:\s+(\d+)", agent).group(1))
+                out.update({"cus": cus, "max_clock_mhz": mhz, "bf16_mfma_tflops_from_cus_and_clock": round(cus * 4096 * mhz / 1e6, 1)})
+                break
+    except Exception as e:                      # the summary is informative only
+        out["rocminfo_error"] = repr(e)[:80]
+    return out
+
+
 def settle_clocks(fn, ms):
     """Keep the GPU busy with the workload for ``ms`` milliseconds.  After an idle period the part
     needs ~20 ms of load before its clocks settle (the first ~100 launches of the headline kernel
@@ -485,7 +506,7 @@ def main():
                      "single_launch": single, "cache_state": "warm: back-to-back launches on the same inputs, no L2 flush",
                      "settle_ms": SETTLE_MS},
         "cpu_baseline": cpu,
-        "device": torch.cuda.get_device_name(0),
+        "device": torch.cuda.get_device_name(0), "device_summary": device_summary(),
     }
     if aux:
         out["aux"] = aux
