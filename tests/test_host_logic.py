@@ -93,7 +93,7 @@ def test_flex_block_mask_matches_oracle():
         a = mb.flex_block_mask(8, ks, 3, bq, block_k=bk)
         b = oracle.flex_block_mask(8, ks, 3, bq, block_k=bk)
         assert torch.equal(a, b)
-    # the shipped CSLA configuration at the last scale: [32, 83] blocks of 128 (survey of SparseFlexAttn)
+    # the shipped CSLA configuration at the last scale: [32, 83] blocks of 128 (SparseFlexAttn, models/sparvar/basic_sparvar.py:55-72)
     m = mb.flex_block_mask(12, [-1, -1, -1, -1, -1, -1, -1, -1, 1, 1, 3, 5, 7], 5, 128)
     assert m.shape == (32, 83) and bool(m[:, 0].all())
 
