@@ -92,3 +92,27 @@ def test_token_lists_random(seed):
     delta, (M, L) = ops.csp_attn_delta(q.cuda(), k.cuda(), v.cuda(), idx.cuda(), counts.cuda())
     d_ref, M_ref, L_ref = oracle.csp_attn_delta(q, k, v, idx, counts)
     assert close(delta, d_ref) and lse_close(M, L, M_ref, L_ref)
+
+
+def test_token_lists_both_workgroup_sizes():
+    """The token-list kernel runs a 192-row group as two 3-wave workgroups in small launches and as one
+    6-wave workgroup in large ones (512 groups and more on a 256-CU part): same rows, same arithmetic, so a
+    (batch, head) slice launched alone must reproduce the large launch bit for bit, and both match the oracle."""
+    from lvar_amd import sparse_attn_ops as ops
+    B, H, Lq, Lk, d = 2, 16, 3072, 333, 64
+    g = torch.Generator().manual_seed(77)
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=77, amp=0.5)
+    G = (Lq + 191) // 192
+    assert B * H * G >= 512
+    idx = torch.randint(0, Lk, (B, H, G, Lk), generator=g, dtype=torch.int32)
+    counts = torch.randint(1, Lk + 1, (B, H, G), generator=g, dtype=torch.int32)
+    o0 = (torch.randn(B, H, Lq, d, generator=g) * 0.5).to(torch.bfloat16)
+    qg, kg, vg, ig, cg, og = q.cuda(), k.cuda(), v.cuda(), idx.cuda(), counts.cuda(), o0.cuda()
+    big = ops.csp_attn(qg, kg, vg, None, ig, cg, og, 1)
+    for (b, h) in ((0, 0), (1, 9)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        small = ops.csp_attn(qg[sl].contiguous(), kg[sl].contiguous(), vg[sl].contiguous(), None,
+                             ig[sl].contiguous(), cg[sl].contiguous(), og[sl].contiguous(), 1)
+        assert torch.equal(small, big[sl]), (b, h)
+        ref = oracle.csp_attn(q[sl], k[sl], v[sl], None, idx[sl], counts[sl], o0[sl], 1)
+        assert close(big[sl], ref), (b, h)
