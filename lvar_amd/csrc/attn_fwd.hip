@@ -30,6 +30,27 @@ namespace lvar {
 #ifndef LVAR_AHEAD
 #define LVAR_AHEAD 4
 #endif
+#ifndef LVAR_EXP_IN_A
+#define LVAR_EXP_IN_A 24   // of the 32 exp2 per lane and tile, how many run next to the QK MFMAs
+#endif
+
+// First S element of softmax slot g: EA elements spread over the NQK steps of the QK phase, the other
+// 32 - EA over the first HB steps of the PV phase; slots before 0 and after the last one are empty.
+template <int NQK, int HB, int EA>
+struct ExpSlots {
+  static constexpr int lo(int g) {
+    return g <= 0 ? 0 : g < NQK ? g * EA / NQK : g < NQK + HB ? EA + (g - NQK) * (32 - EA) / HB : 32;
+  }
+};
+
+// f(integral_constant<int, i>) for i = LO .. HI-1, unrolled at compile time
+template <int LO, int HI, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (LO < HI) {
+    f(std::integral_constant<int, LO>{});
+    static_for<LO + 1, HI>(f);
+  }
+}
 static constexpr float RESCALE_TAU = 8.0f;
 static constexpr float NEG_BIG = -1.0e30f;
 
@@ -155,6 +176,30 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     // Written as inline assembly so that the compiler does not serialise later LDS reads of the
     // OTHER buffers behind these fills; completion is awaited with vmcnt(0) before the barrier.
     auto issue = [&](const i32x4& rsrc, int srb, bool is_v, const int (&rows)[NR], uint32_t dst) {
+      // Block lists, tile fully inside K/V: the rows of a tile are consecutive, so the per-lane byte
+      // offset (row within the first instruction, swizzled chunk: the swizzle does not depend on the
+      // slot) is a constant and tile and slot only move a scalar offset.
+      const int row0 = __builtin_amdgcn_readfirstlane(rows[0]);  // wave-uniform for block lists
+      if (MODE == MODE_BLOCK && row0 + 64 <= p.Lk) {
+        const int trow0 = wave * RPI + lrow;
+        const int voff = trow0 * srb + ((lcs ^ (is_v ? Swz<D>::fv(trow0) : Swz<D>::fk(trow0))) << 4);
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+          const int i = wave + s * NWAVES;
+          if ((NI % NWAVES == 0) || i < NI) {
+            const int soff = (row0 + s * NWAVES * RPI) * srb;
+            const uint32_t m0v = dst + i * 1024;
+            asm volatile(
+                "s_mov_b32 m0, %0\n\t"
+                "s_nop 0\n\t"
+                "buffer_load_dwordx4 %1, %2, %3 offen lds"
+                :
+                : "s"(m0v), "v"(voff), "s"(rsrc), "s"(soff)
+                : "memory");
+          }
+        }
+        return;
+      }
 #pragma unroll
       for (int s = 0; s < SLOTS; s++) {
         const int i = wave + s * NWAVES;
@@ -320,9 +365,9 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       if (t + 3 < T) finish_rows(t + 3, raw, rows_n, nv3);
       if (t + 4 < T) prefetch_raw(t + 4, raw);
       // The block below is software-pipelined by hand; sched_barrier(0) after every step stops the
-      // compiler from regrouping it.  Phase A: QK MFMA j | K-fragment read j+4 | exp2 of two
-      // elements of S(t).  Phase B: PV MFMA j | the two transposing V reads of MFMA j+4 | a slice
-      // of the row-maximum reduction of S(t+1).
+      // compiler from regrouping it.  Phase A: QK MFMA j | K-fragment read j+4 | softmax slot j of
+      // S(t).  Phase B: PV MFMA j | the two transposing V reads of MFMA j+4 | the last softmax slots
+      // of S(t) (first half) or a slice of the row-maximum reduction of S(t+1) (second half).
       constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = LVAR_AHEAD;
       const char* kbuf = smem + (1 - PAR) * TILE;
       const char* vbuf = smem + (2 + PAR) * TILE;
@@ -336,67 +381,90 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
         bf16x4 hi = lds_read_tr(a + 8 * ROWB);
         return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       };
-#pragma unroll
-      for (int i = 0; i < 16; i++) { n0[i] = 0.f; n1[i] = 0.f; }
       bf16x8 frag[NQK > NPV ? NQK : NPV];
       uint32_t pw[16];
       const float negm = -m_ref;
       float la = 0.f, lb = 0.f;
+      // The softmax of S(t) runs as a three-stage pipeline over the MFMA steps so that no vector instruction
+      // waits for the one before it: step g scales the elements of slot g, takes exp2 of slot g-1 and
+      // adds / packs slot g-2.  Slots: EA elements over the QK steps, the rest over the first half of the
+      // PV steps (quarter kb of P is complete before PV step kb * MTD needs it); the row maximum of
+      // S(t+1) goes next to the second half of the PV steps.
+      auto st_scale = [&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        if constexpr (e < 16) c0[e] = fmaf(c0[e], c, negm); else c1[e - 16] = fmaf(c1[e - 16], c, negm);
+      };
+      auto st_exp = [&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        if constexpr (e < 16) c0[e] = fast_exp2(c0[e]); else c1[e - 16] = fast_exp2(c1[e - 16]);
+      };
+      auto st_sum = [&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        float r;
+        if constexpr (e < 16) r = c0[e]; else r = c1[e - 16];
+        if constexpr (e & 1) {
+          lb += r;
+          float prev;
+          if constexpr (e < 16) prev = c0[e - 1]; else prev = c1[e - 17];
+          pw[e >> 1] = pack_bf16(prev, r);
+        } else {
+          la += r;
+        }
+      };
+      using Sch = ExpSlots<2 * KS, (LSE_ONLY ? 0 : 4 * MTD) / 2, LSE_ONLY ? 32 : LVAR_EXP_IN_A>;
+      auto softmax_step = [&](auto gc) {
+        constexpr int g = decltype(gc)::value;
+        static_for<Sch::lo(g - 2), Sch::lo(g - 1)>(st_sum);
+        static_for<Sch::lo(g - 1), Sch::lo(g)>(st_exp);
+        static_for<Sch::lo(g), Sch::lo(g + 1)>(st_scale);
+      };
+      constexpr int HB = NPV / 2;
 #pragma unroll
       for (int j = 0; j < AHEAD; j++) frag[j] = kread(j);
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int j = 0; j < NQK; j++) {
-        if (j + AHEAD < NQK) frag[j + AHEAD] = kread(j + AHEAD);
-        if (j & 1) n1 = mfma32(frag[j], qf[j >> 1], n1);
+      static_for<0, NQK>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        if constexpr (j + AHEAD < NQK) frag[j + AHEAD] = kread(j + AHEAD);
+        // the first MFMA of each accumulator takes the constant 0 as its addend (no register clearing)
+        if constexpr (j == 0) n0 = mfma32(frag[j], qf[0], f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0});
+        else if constexpr (j == 1) n1 = mfma32(frag[j], qf[0], f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0});
+        else if constexpr (j & 1) n1 = mfma32(frag[j], qf[j >> 1], n1);
         else n0 = mfma32(frag[j], qf[j >> 1], n0);
-        // exp2 share of this step: 32 / NQK element pairs of S(t)
-#pragma unroll
-        for (int u = 0; u < 16 / NQK; u++) {
-          const int w = j * (16 / NQK) + u;  // pair index 0..15: elements 2w, 2w+1
-          float x0, x1;
-          if (w < 8) { x0 = c0[2 * w]; x1 = c0[2 * w + 1]; } else { x0 = c1[2 * w - 16]; x1 = c1[2 * w - 15]; }
-          x0 = fast_exp2(fmaf(x0, c, negm));
-          x1 = fast_exp2(fmaf(x1, c, negm));
-          la += x0;
-          lb += x1;
-          pw[w] = pack_bf16(x0, x1);
-        }
+        softmax_step(jc);
         __builtin_amdgcn_sched_barrier(0);
-      }
-      lsum += la + lb;
+      });
       float ma = -INFINITY, mb = -INFINITY;
       if (!LSE_ONLY) {
         bf16x8 pb[4];
 #pragma unroll
-        for (int kb = 0; kb < 4; kb++) {
-          u32x4 u = {pw[4 * kb], pw[4 * kb + 1], pw[4 * kb + 2], pw[4 * kb + 3]};
-          pb[kb] = __builtin_bit_cast(bf16x8, u);
-        }
-#pragma unroll
         for (int j = 0; j < AHEAD; j++) frag[j] = vread(j);
         __builtin_amdgcn_sched_barrier(0);
         if (MASKED) mask_tile(n0, n1, nv1);
-#pragma unroll
-        for (int j = 0; j < NPV; j++) {
-          if (j + AHEAD < NPV) frag[j + AHEAD] = vread(j + AHEAD);
+        static_for<0, NPV>([&](auto jc) {
+          constexpr int j = decltype(jc)::value;
+          if constexpr (j + AHEAD < NPV) frag[j + AHEAD] = vread(j + AHEAD);
+          if constexpr (j % MTD == 0) {
+            constexpr int kb = j / MTD;
+            u32x4 u = {pw[4 * kb], pw[4 * kb + 1], pw[4 * kb + 2], pw[4 * kb + 3]};
+            pb[kb] = __builtin_bit_cast(bf16x8, u);
+          }
           oacc[j % MTD] = mfma32(frag[j], pb[j / MTD], oacc[j % MTD]);
-          // row-maximum share: spread the 32 elements of S(t+1) over the steps after the first AHEAD
-          constexpr int MSTEPS = NPV - AHEAD;
-          if (j >= AHEAD) {
-            const int e0 = (j - AHEAD) * 16 / MSTEPS, e1 = (j - AHEAD + 1) * 16 / MSTEPS;
+          softmax_step(std::integral_constant<int, NQK + j>{});
+          if constexpr (j >= HB) {
+            constexpr int e0 = (j - HB) * 16 / (NPV - HB), e1 = (j - HB + 1) * 16 / (NPV - HB);
 #pragma unroll
-            for (int e = e0; e < e1; e++) {
-              ma = fmaxf(fmaxf(ma, n0[e]), n1[e]);
-            }
+            for (int e = e0; e < e1; e++) ma = fmaxf(fmaxf(ma, n0[e]), n1[e]);
           }
           __builtin_amdgcn_sched_barrier(0);
-        }
+        });
       } else {
+        softmax_step(std::integral_constant<int, NQK>{});
+        softmax_step(std::integral_constant<int, NQK + 1>{});
         if (MASKED) mask_tile(n0, n1, nv1);
 #pragma unroll
         for (int e = 0; e < 16; e++) ma = fmaxf(fmaxf(ma, n0[e]), n1[e]);
       }
+      lsum += la + lb;
       const float mx = xhalf_max(fmaxf(ma, mb));
       __builtin_amdgcn_s_waitcnt(0x0f70);
       __syncthreads();

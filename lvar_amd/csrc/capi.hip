@@ -1,6 +1,5 @@
 // extern "C" entry points declared in include/lvar_sparse_attn.h: argument validation and
 // parameter packing; all device work is in attn_fwd.hip / colsum.hip.
-#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include "../../include/lvar_sparse_attn.h"
@@ -28,31 +27,16 @@ bool shape_ok(int B, int H, int Lq, int Lk, float scale) {
   return B > 0 && H > 0 && Lq > 0 && Lk > 0 && std::isfinite(scale) && scale > 0.f;
 }
 
-// Compute units of the current device (cached per device; 256 on MI355X).
-int cu_count() {
-  static std::atomic<int> cached[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return 256;
-  std::atomic<int>& slot = cached[dev & 63];
-  int n = slot.load(std::memory_order_relaxed);
-  if (n == 0) {
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    slot.store(n, std::memory_order_relaxed);
-  }
-  return n;
-}
-
-// Waves per workgroup of the token-list kernel.  A 192-row group is one 6-wave workgroup (one per CU)
-// or two 3-wave workgroups (two per CU, twice the K/V fills): the small ones win while the 6-wave
-// launch has fewer than two workgroups per CU, the large one beyond.  LVAR_CSP_WAVES=2|3|6 overrides.
-int gather_waves(int64_t groups) {
-  static int forced = [] {
+// Waves per workgroup of the token-list kernel.  A 192-row group runs as one 6-wave workgroup (one per
+// CU); two 3-wave workgroups per group double the K/V fills and spill registers, and are only taken when
+// the group size is not a multiple of 192 rows.  LVAR_CSP_WAVES=2|3|6 overrides the first choice.
+int gather_waves() {
+  static int v = [] {
     const char* e = std::getenv("LVAR_CSP_WAVES");
-    const int n = e ? std::atoi(e) : 0;
-    return (n == 2 || n == 3 || n == 6) ? n : 0;
+    const int n = e ? std::atoi(e) : 6;
+    return (n == 2 || n == 3 || n == 6) ? n : 6;
   }();
-  if (forced) return forced;
-  return groups < 2 * (int64_t)cu_count() ? 3 : 6;
+  return v;
 }
 
 void fill_qkv(AttnParams& p, const lvar_tensor_t& q, const lvar_tensor_t& k, const lvar_tensor_t& v) {
@@ -133,7 +117,7 @@ static int csp_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_te
   p.list_len = (int)(idx_row_stride > 0x7fffffff ? 0x7fffffff : idx_row_stride);
   p.group_rows = group_rows;
   p.up_src = up_src; p.up_dst = up_dst;
-  int nw = gather_waves((int64_t)B * H * G);
+  int nw = gather_waves();
   while (group_rows % (nw * 32) != 0) nw = (nw == 6) ? 3 : (nw == 3 ? 2 : 1);
   if (nw == 1) {
     if (group_rows % 64 == 0) nw = 2; else return LVAR_EUNSUPPORTED;
