@@ -31,14 +31,14 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel
 # of known size; the summaries are under profiles/.  None = not measured for that workload.
 MEASURED_TRAFFIC = {
-    # profiles/attn_fwd_block_sparse_infinity2b_1024_last_scale_25pct.txt: FETCH 100940 KiB x 2.0 + WRITE 33792 KiB x 1.0
-    "block_sparse_25": 241.3e6,
-    # profiles/attn_fwd_dense_infinity2b_1024_last_scale.txt: FETCH 100690 KiB x 2.0 + WRITE 33792 KiB x 1.0
+    # profiles/attn_fwd_block_sparse_infinity2b_1024_last_scale_25pct.txt: FETCH 100990 KiB x 2.0 + WRITE 33741 KiB x 1.0
+    "block_sparse_25": 241.4e6,
+    # profiles/attn_fwd_dense_infinity2b_1024_last_scale.txt: FETCH 100700 KiB x 2.0 + WRITE 33792 KiB x 1.0
     "dense": 240.8e6,
     # profiles/colsum_infinity2b_1024_last_scale.txt: FETCH 65610 KiB x 2.0 + WRITE 28990 KiB x 1.0
     "colsum": 164.1e6,
-    # profiles/attn_fwd_token_list_infinity2b_1024_last_scale_top20pct.txt: FETCH 141390 KiB x 2.0 + WRITE 32768 KiB x 1.0
-    "csp": 323.1e6,
+    # profiles/attn_fwd_token_list_infinity2b_1024_last_scale_top20pct.txt: FETCH 141250 KiB x 2.0 + WRITE 32716 KiB x 1.0
+    "csp": 322.8e6,
 }
 
 
