@@ -65,16 +65,32 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
   const int lrow = lane / CPR, lcs = lane % CPR;
 
   // global->LDS fill of stage s (Q rows s*64 .. +63, clamped to Lq-1, chunk-swizzled; lse2 by wave 0)
+  // lane offset of a Q fill: row within the first instruction of this wave, swizzled chunk (the swizzle
+  // repeats every 16 rows, i.e. does not depend on the slot: instruction i = wave + 4 * slot covers rows
+  // i * RPI ..)
+  const int fill_trow0 = wave * RPI + lrow;
+  const int fill_voff = fill_trow0 * q_srb + ((lcs ^ ((fill_trow0 / (256 / ROWB)) & (CPR - 1))) << 4);
   auto issue_stage = [&](int s) {
     const uint32_t dst = lds0 + (s & (NSTAGE - 1)) * QTILE;
+    if (s * 64 + 64 <= p.Lq) {
+      // all 64 rows exist: constant lane offset, stage and slot move the scalar offset
 #pragma unroll
-    for (int sl = 0; sl < SLOTS; sl++) {
-      const int i = wave + sl * 4;
-      const int trow = i * RPI + lrow;
-      const int grow = min(s * 64 + trow, p.Lq - 1);
-      const int voff = grow * q_srb + ((lcs ^ ((trow / (256 / ROWB)) & (CPR - 1))) << 4);
-      const uint32_t m0v = dst + i * 1024;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(m0v), "v"(voff), "s"(qrsrc) : "memory");
+      for (int sl = 0; sl < SLOTS; sl++) {
+        const int i = wave + sl * 4;
+        const int soff = (s * 64 + sl * 4 * RPI) * q_srb;
+        const uint32_t m0v = dst + i * 1024;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(m0v), "v"(fill_voff), "s"(qrsrc), "s"(soff) : "memory");
+      }
+    } else {
+#pragma unroll
+      for (int sl = 0; sl < SLOTS; sl++) {
+        const int i = wave + sl * 4;
+        const int trow = i * RPI + lrow;
+        const int grow = min(s * 64 + trow, p.Lq - 1);
+        const int voff = grow * q_srb + ((lcs ^ ((trow / (256 / ROWB)) & (CPR - 1))) << 4);
+        const uint32_t m0v = dst + i * 1024;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(m0v), "v"(voff), "s"(qrsrc) : "memory");
+      }
     }
     if (wave == 0) {
       const int voff = min(s * 64 + lane, p.Lq - 1) * 4;
@@ -159,8 +175,7 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
     const char* qb = smem + ((u >> 1) & (NSTAGE - 1)) * QTILE + (u & 1) * 32 * ROWB;
     constexpr int AHEAD = 3;
     bf16x8 frag[KS];
-#pragma unroll
-    for (int i = 0; i < 16; i++) { n0a[i] = 0.f; n1a[i] = 0.f; }
+    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};   // constant addend of the first MFMA
 #pragma unroll
     for (int j = 0; j < AHEAD && j < KS; j++) frag[j] = *(const bf16x8*)(qb + (kbase_l ^ (j << 5)));
     if (have_prev) {
@@ -170,21 +185,47 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
 #pragma unroll
       for (int j = 0; j < 4; j++) lse[j] = *(const f32x4*)(ll + j * 32);
       float pa = 0.f, pb = 0.f;
+      // probabilities of tile u-1 as a three-stage pipeline over the MFMA steps (scale | exp2 | add), 16 / KS
+      // accumulator indices of both key tiles per step, so that no vector instruction waits for the last one
+      constexpr int EPS = 16 / KS;
+      float xs0[16], xs1[16];
+      auto st_scale = [&](int g) {
+#pragma unroll
+        for (int e = 0; e < EPS; e++) {
+          const int i = g * EPS + e;
+          xs0[i] = fmaf(c0[i], c, -lse[i >> 2][i & 3]);
+          xs1[i] = fmaf(c1[i], c, -lse[i >> 2][i & 3]);
+        }
+      };
+      auto st_exp = [&](int g) {
+#pragma unroll
+        for (int e = 0; e < EPS; e++) {
+          const int i = g * EPS + e;
+          xs0[i] = fast_exp2(xs0[i]);
+          xs1[i] = fast_exp2(xs1[i]);
+        }
+      };
+      auto st_add = [&](int g) {
+#pragma unroll
+        for (int e = 0; e < EPS; e++) {
+          const int i = g * EPS + e;
+          pa += xs0[i];
+          pb += xs1[i];
+        }
+      };
+      st_scale(0);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
         if (ks + AHEAD < KS) frag[ks + AHEAD] = *(const bf16x8*)(qb + (kbase_l ^ ((ks + AHEAD) << 5)));
-        n0a = mfma32(frag[ks], kf[0][ks], n0a);
-        n1a = mfma32(frag[ks], kf[1][ks], n1a);
-        // share of the exp work: 16 / KS accumulator indices of both key tiles
-#pragma unroll
-        for (int e = 0; e < 16 / KS; e++) {
-          const int i = ks * (16 / KS) + e;
-          pa += fast_exp2(fmaf(c0[i], c, -lse[i >> 2][i & 3]));
-          pb += fast_exp2(fmaf(c1[i], c, -lse[i >> 2][i & 3]));
-        }
+        n0a = mfma32(frag[ks], kf[0][ks], ks == 0 ? zero : n0a);
+        n1a = mfma32(frag[ks], kf[1][ks], ks == 0 ? zero : n1a);
+        if (ks >= 1) st_add(ks - 1);
+        st_exp(ks);
+        if (ks + 1 < KS) st_scale(ks + 1);
         __builtin_amdgcn_sched_barrier(0);
       }
+      st_add(KS - 1);
       acc[0] += pa;
       acc[1] += pb;
       const int qend = up * 32 + 32;
@@ -193,8 +234,8 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
         if (ks + AHEAD < KS) frag[ks + AHEAD] = *(const bf16x8*)(qb + (kbase_l ^ ((ks + AHEAD) << 5)));
-        n0a = mfma32(frag[ks], kf[0][ks], n0a);
-        n1a = mfma32(frag[ks], kf[1][ks], n1a);
+        n0a = mfma32(frag[ks], kf[0][ks], ks == 0 ? zero : n0a);
+        n1a = mfma32(frag[ks], kf[1][ks], ks == 0 ? zero : n1a);
       }
     }
   };
