@@ -76,7 +76,8 @@ int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* 
  * [B,H,G,idx_row_stride] (row stride in elements, >= max count), counts int32 [B,H,G]
  * contiguous, clamped to [0, idx_row_stride].  Indices outside [0,Lk) are clamped.  count == 0 leaves o = o_accum,
  * M = -inf, L = 1.  o_accum may be NULL (treated as zero) and may alias o.
- * group_rows must be a multiple of 32 (the reference uses 192).
+ * group_rows must be a multiple of 32 (the reference uses 192).  Gathered rows are addressed with a 24-bit
+ * multiply: Lk <= 2^24 and K/V row strides below 2^23 elements, else LVAR_EUNSUPPORTED.
  * Replaces sattn_triton.csp_attn (kernels/sparse_attn/triton/attn_csp.py:215-265) and
  * torch.ops.chipmunk.csp_attn (kernels/chipmunk/csrc/chipmunk.cu:59,
  * kernels/chipmunk/csrc/attn/csp_attn.cu:318-433).

@@ -169,7 +169,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       } else {
         nvalid = min(64, count - (t << 6));
 #pragma unroll
-        for (int s = 0; s < NR; s++) rows[s] = raw[s];
+        for (int s = 0; s < NR; s++) rows[s] = max(0, min(raw[s], p.Lk - 1));   // clamped once, used by the K and the V fill
       }
     };
     // Issue the global->LDS loads of one tile (K or V) into the LDS buffer at byte address `dst`.
@@ -206,8 +206,14 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
         if ((NI % NWAVES == 0) || i < NI) {
           const int trow = i * RPI + lrow;
           const int chunk = lcs ^ (is_v ? Swz<D>::fv(trow) : Swz<D>::fk(trow));
-          const int grow = max(0, min((MODE == MODE_GATHER) ? rows[s < NR ? s : 0] : rows[0] + trow, p.Lk - 1));
-          const int voff = grow * srb + chunk * 16;
+          int voff;
+          if (MODE == MODE_GATHER) {
+            // token rows and row strides are below 2^24 (checked on the host): one full-rate 24-bit multiply-add
+            voff = (int)(((unsigned)rows[s < NR ? s : 0] & 0xffffffu) * ((unsigned)srb & 0xffffffu) + (unsigned)(chunk * 16));
+          } else {
+            const int grow = max(0, min(rows[0] + trow, p.Lk - 1));
+            voff = grow * srb + chunk * 16;
+          }
           const uint32_t m0v = dst + i * 1024;
           asm volatile(
               "s_mov_b32 m0, %0\n\t"

@@ -102,6 +102,8 @@ static int csp_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_te
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
   if (o_accum.ptr && !view_ok(o_accum)) return LVAR_EINVAL;
   if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
+  // gathered rows are addressed with a 24-bit multiply: token index and row stride in bytes below 2^24
+  if (Lk > (1 << 24) || k.stride_row * 2 >= (1 << 24) || v.stride_row * 2 >= (1 << 24)) return LVAR_EUNSUPPORTED;
   if (!indices || !counts || G <= 0 || idx_row_stride <= 0) return LVAR_EINVAL;
   if (group_rows <= 0 || group_rows % 32 != 0 || (int64_t)G * group_rows < Lq) return LVAR_EINVAL;
   AttnParams p{};
