@@ -180,7 +180,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       // offset (row within the first instruction, swizzled chunk: the swizzle does not depend on the
       // slot) is a constant and tile and slot only move a scalar offset.
       const int row0 = __builtin_amdgcn_readfirstlane(rows[0]);  // wave-uniform for block lists
-      if (MODE == MODE_BLOCK && row0 + 64 <= p.Lk) {
+      if (MODE == MODE_BLOCK && row0 >= 0 && row0 <= p.Lk - 64) {   // anything else takes the clamped path below
         const int trow0 = wave * RPI + lrow;
         const int voff = trow0 * srb + ((lcs ^ (is_v ? Swz<D>::fv(trow0) : Swz<D>::fk(trow0))) << 4);
 #pragma unroll
