@@ -76,3 +76,31 @@ def load() -> C.CDLL:
 def check(status: int, where: str) -> None:
     if status != 0:
         raise LvarError(status, where, load().lvar_status_string(status).decode())
+
+
+_binding = False      # False: not tried yet; None: not available
+
+
+def torch_binding():
+    """The compiled torch binding (``_lvar_torch.so`` next to this file), bound to the loaded C-ABI library, or
+    None when it is not built, does not load, or ``LVAR_AMD_NO_TORCH_BINDING`` is set.  It only shortens the
+    host side of ``dense_attn``; every call it declines goes through the ctypes path."""
+    global _binding
+    if _binding is not False:
+        return _binding
+    _binding = None
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lvar_torch.so")
+    if os.environ.get("LVAR_AMD_NO_TORCH_BINDING") or not os.path.exists(path):
+        return None
+    try:
+        import importlib.util
+        import torch  # noqa: F401  (the module links against libtorch)
+        spec = importlib.util.spec_from_file_location("_lvar_torch", path)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        mod.bind(C.cast(load().lvar_dense_attn_fwd, C.c_void_p).value)
+        _binding = mod
+    except Exception:          # a stale or incompatible module must not take the ctypes path down with it
+        _binding = None
+    return _binding
+

@@ -1,9 +1,10 @@
-"""Build the C-ABI shared library ``lvar_amd/liblvar_sparse_attn.so`` for gfx950 with hipcc.
+"""Build the C-ABI shared library ``lvar_amd/liblvar_sparse_attn.so`` for gfx950 with hipcc, and the
+compiled torch binding ``lvar_amd/_lvar_torch.so`` (host code only, g++ against the torch headers).
 
     python -m lvar_amd.build
 
-hipcc cross-compiles without a GPU.  The library is built in-tree so that it travels with
-the source tree; nothing is installed into site-packages.
+hipcc cross-compiles without a GPU.  Both are built in-tree so that they travel with the source tree;
+nothing is installed into site-packages.
 """
 from __future__ import annotations
 
@@ -64,6 +65,39 @@ def build_library(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+BINDING_NAME = "_lvar_torch"
+BINDING_PATH = os.path.join(HERE, BINDING_NAME + ".so")
+
+
+def build_torch_binding(verbose: bool = False) -> str:
+    """Compile ``csrc/torch_binding.cpp`` (the compiled fast path of ``dense_attn``) into a Python extension
+    module.  Host code only: g++ with torch's include paths; the module receives the address of the C-ABI
+    entry point at run time, so it does not link the HIP library.  Always rebuilds."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+    cxx = shutil.which("g++")
+    if cxx is None:
+        raise RuntimeError("g++ not found; it is needed for the torch binding")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    inc = ce.include_paths() + [sysconfig.get_paths()["include"], os.path.join(rocm, "include")]
+    tmp = BINDING_PATH + ".tmp"
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", f"-DTORCH_EXTENSION_NAME={BINDING_NAME}", "-D__HIP_PLATFORM_AMD__",
+           "-DUSE_ROCM", "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           *["-I" + i for i in inc], os.path.join(CSRC, "torch_binding.cpp"), "-o", tmp,
+           "-L" + tlib, "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python", "-Wl,-rpath," + tlib]
+    out = _run(cmd)
+    os.replace(tmp, BINDING_PATH)
+    if verbose:
+        if out.strip():
+            print(out)
+        print("built", BINDING_PATH)
+    return BINDING_PATH
+
+
 if __name__ == "__main__":
     build_library(verbose=True)
+    build_torch_binding(verbose=True)
     sys.exit(0)

@@ -126,6 +126,11 @@ def _dense_launch(q, k, v, scale, want_o=True, want_ml=True, want_lse2=False):
 def dense_attn(q, k, v, scale=None):
     """Dense flash attention, ``(o, (M, L))`` (reference ``dense_attn``, sparse_attn_ops.py:21-59,
     Triton-provider return convention: ``lse`` is the tuple ``(M, L)``, each ``[B,H,Lq,1]``)."""
+    fast = _lib.torch_binding()
+    if fast is not None:
+        r = fast.fast_dense_attn(q, k, v, scale)      # None unless the inputs are the plain contiguous bf16 case
+        if r is not None:
+            return r[0], (r[1], r[2])
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
     _check_qkv(q, k, v)
     o, M, L, _ = _dense_launch(q, k, v, scale)

@@ -115,3 +115,18 @@ def test_missing_library_is_an_import_error(monkeypatch):
     monkeypatch.setenv("LVAR_AMD_LIB", "/nonexistent/liblvar.so")
     with pytest.raises(ImportError, match="no CPU or PyTorch fallback"):
         _lib.load()
+
+
+def test_torch_binding_loads_and_declines_cpu_tensors(lib):
+    """The compiled fast path of dense_attn is optional: when it is built it must load, bind to the C-ABI
+    library and hand anything but plain device tensors back to the general path (None)."""
+    import os
+    import torch
+    from lvar_amd import _lib
+    path = os.path.join(os.path.dirname(_lib.__file__), "_lvar_torch.so")
+    if not os.path.exists(path):
+        pytest.skip("torch binding not built")
+    mod = _lib.torch_binding()
+    assert mod is not None and hasattr(mod, "fast_dense_attn") and hasattr(mod, "bind")
+    x = torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16)
+    assert mod.fast_dense_attn(x, x, x, None) is None            # CPU tensors: not its case, and no GPU call is made

@@ -270,3 +270,32 @@ def test_window_key_scores_and_scalekv_selection():
                     assert len(rest) == 50
                     thr = torch.topk(sc[b, h], 50).values[-1]
                     assert bool((sc[b, h, rest] >= thr).all())
+
+
+def test_compiled_dense_binding_matches_ctypes_path():
+    """dense_attn through the compiled torch binding (when built) and through the ctypes path: same bits;
+    strided, misaligned or wrongly typed inputs fall through to the general path with its behaviour."""
+    from lvar_amd import _lib, sparse_attn_ops as ops
+    mod = _lib.torch_binding()
+    if mod is None:
+        pytest.skip("torch binding not built")
+    q, k, v = make_qkv(2, 3, 200, 333, 128, seed=5, amp=0.5)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    for scale in (None, 0.07):
+        fast = mod.fast_dense_attn(qg, kg, vg, scale)
+        assert fast is not None
+        o, M, L, _ = ops._dense_launch(qg, kg, vg, scale)
+        assert torch.equal(fast[0], o) and torch.equal(fast[1], M) and torch.equal(fast[2], L)
+        assert fast[1].shape == (2, 3, 200, 1) and fast[2].shape == (2, 3, 200, 1)
+        o2, (M2, L2) = ops.dense_attn(qg, kg, vg, scale)
+        assert torch.equal(o2, o) and torch.equal(M2, M) and torch.equal(L2, L)
+    # not the plain case: strided views, fp16, mismatched shapes
+    assert mod.fast_dense_attn(qg.transpose(1, 2), kg, vg, None) is None
+    assert mod.fast_dense_attn(qg.half(), kg.half(), vg.half(), None) is None
+    assert mod.fast_dense_attn(qg, kg, vg[:, :, :100], None) is None
+    qs = qg.transpose(1, 2).contiguous().transpose(1, 2)          # [B,H,L,d] view of a [B,L,H,d] buffer
+    o3, _ = ops.dense_attn(qs, kg, vg, None)
+    o_ref, _, _, _ = ops._dense_launch(qg, kg, vg, None)
+    assert torch.equal(o3, o_ref)
+    with pytest.raises((TypeError, ValueError)):
+        ops.dense_attn(qg.half(), kg.half(), vg.half())
