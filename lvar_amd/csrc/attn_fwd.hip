@@ -181,6 +181,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       // slot) is a constant and tile and slot only move a scalar offset.
       const int row0 = __builtin_amdgcn_readfirstlane(rows[0]);  // wave-uniform for block lists
       if (MODE == MODE_BLOCK && row0 >= 0 && row0 <= p.Lk - 64) {   // anything else takes the clamped path below
+        static_assert(MODE != MODE_BLOCK || (NWAVES * RPI) % 16 == 0, "slots of one wave must be a swizzle period (16 rows) apart");
         const int trow0 = wave * RPI + lrow;
         const int voff = trow0 * srb + ((lcs ^ (is_v ? Swz<D>::fv(trow0) : Swz<D>::fk(trow0))) << 4);
 #pragma unroll

@@ -68,6 +68,7 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
   // lane offset of a Q fill: row within the first instruction of this wave, swizzled chunk (the swizzle
   // repeats every 16 rows, i.e. does not depend on the slot: instruction i = wave + 4 * slot covers rows
   // i * RPI ..)
+  static_assert((4 * RPI) % 16 == 0, "slots of one wave must be a swizzle period (16 rows) apart");
   const int fill_trow0 = wave * RPI + lrow;
   const int fill_voff = fill_trow0 * q_srb + ((lcs ^ ((fill_trow0 / (256 / ROWB)) & (CPR - 1))) << 4);
   auto issue_stage = [&](int s) {
