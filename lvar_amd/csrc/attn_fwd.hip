@@ -3,6 +3,7 @@
 //
 // Work decomposition
 //   workgroup  = NWAVES waves, 32 query rows per wave, all waves share the K/V tiles in LDS
+//                (token lists: 8 waves = 6 computing waves + 2 waves that only fetch, see NPROD)
 //   wave       = S^T[64 keys x 32 queries] = K_tile . Q^T with 32x32x16 bf16 MFMA (K rows are
 //                the A operand read from LDS, Q^T is the B operand held in registers), so a
 //                lane owns ONE query column: the softmax row max / sum are in-register
@@ -70,15 +71,22 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   // The body is compiled for the device only: the host pass just needs the launch stub, and it
   // silently drops the stub when the body uses the LDS-DMA builtins.
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int WGROWS = NWAVES * 32;
+  // Token lists with 8 waves: waves 0..5 compute (one 192-row group), waves 6 and 7 only fetch -- they read
+  // the list, form the gather addresses and issue every K/V fill.  One 6-wave group fills 6 of the 8 wave
+  // slots of a CU; the two fetch waves take the idle ones and the compute waves lose ~10 % of their
+  // instructions.  Everywhere else all waves do both.
+  constexpr int NPROD = (MODE == MODE_GATHER && NWAVES == 8) ? 2 : 0;
+  constexpr int NCOMP = NWAVES - NPROD;     // computing waves, 32 query rows each
+  constexpr int FW = NPROD ? NPROD : NWAVES;  // waves that issue the fills
+  constexpr int WGROWS = NCOMP * 32;
   constexpr int KS = D / 16, MTD = D / 32;
   constexpr int ROWB = Swz<D>::ROWB, CPR = Swz<D>::CPR;
   constexpr int RPI = 1024 / ROWB;          // rows filled by one 64-lane x 16 B load
   constexpr int NI = 64 / RPI;              // loads per 64-row tile
-  constexpr int SLOTS = (NI + NWAVES - 1) / NWAVES;
+  constexpr int SLOTS = (NI + FW - 1) / FW;
   constexpr int TILE = 64 * ROWB;
   constexpr int OSTR = D * 2 + 16;  // epilogue transpose buffer row stride (bytes)
-  static_assert(NWAVES * 32 * OSTR <= 4 * TILE, "epilogue buffer must fit in the K/V buffers");
+  static_assert(NCOMP * 32 * OSTR <= 4 * TILE, "epilogue buffer must fit in the K/V buffers");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   // LDS map: K buffers at 0 and TILE, V buffers at 2*TILE and 3*TILE
 
@@ -92,6 +100,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, r = lane & 31;
+  const int fwave = NPROD ? wave - NCOMP : wave;   // index among the filling waves (negative: this wave does not fill)
   const int q0 = qt * WGROWS;
   const int g = q0 / p.group_rows;
 
@@ -155,7 +164,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       } else {
 #pragma unroll
         for (int s = 0; s < SLOTS; s++) {
-          const int trow = (wave + s * NWAVES) * RPI + lrow;
+          const int trow = (fwave + s * FW) * RPI + lrow;
           const int pos = (t << 6) + trow;
           raw[s] = (pos < count && trow < 64) ? list[pos] : 0;
         }
@@ -181,14 +190,14 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       // slot) is a constant and tile and slot only move a scalar offset.
       const int row0 = __builtin_amdgcn_readfirstlane(rows[0]);  // wave-uniform for block lists
       if (MODE == MODE_BLOCK && row0 >= 0 && row0 <= p.Lk - 64) {   // anything else takes the clamped path below
-        static_assert(MODE != MODE_BLOCK || (NWAVES * RPI) % 16 == 0, "slots of one wave must be a swizzle period (16 rows) apart");
-        const int trow0 = wave * RPI + lrow;
+        static_assert(MODE != MODE_BLOCK || (FW * RPI) % 16 == 0, "slots of one wave must be a swizzle period (16 rows) apart");
+        const int trow0 = fwave * RPI + lrow;
         const int voff = trow0 * srb + ((lcs ^ (is_v ? Swz<D>::fv(trow0) : Swz<D>::fk(trow0))) << 4);
 #pragma unroll
         for (int s = 0; s < SLOTS; s++) {
-          const int i = wave + s * NWAVES;
-          if ((NI % NWAVES == 0) || i < NI) {
-            const int soff = (row0 + s * NWAVES * RPI) * srb;
+          const int i = fwave + s * FW;
+          if ((NI % FW == 0) || i < NI) {
+            const int soff = (row0 + s * FW * RPI) * srb;
             const uint32_t m0v = dst + i * 1024;
             asm volatile(
                 "s_mov_b32 m0, %0\n\t"
@@ -203,8 +212,8 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       }
 #pragma unroll
       for (int s = 0; s < SLOTS; s++) {
-        const int i = wave + s * NWAVES;
-        if ((NI % NWAVES == 0) || i < NI) {
+        const int i = fwave + s * FW;
+        if ((NI % FW == 0) || i < NI) {
           const int trow = i * RPI + lrow;
           const int chunk = lcs ^ (is_v ? Swz<D>::fv(trow) : Swz<D>::fk(trow));
           int voff;
@@ -226,6 +235,41 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
         }
       }
     };
+
+    // valid keys of tile t of a token list (only the last tile can be ragged)
+    auto nvalid_gather = [&](int t) { return max(0, min(64, count - (t << 6))); };
+
+    if (NPROD && wave >= NCOMP) {
+      // ---- fetch waves: the fill schedule of the loop below and nothing else; one barrier per tile ----
+      int rows_v[NR], rows_k[NR], rows_n[NR], raw[NR], rows0[NR];
+      int nv_unused;
+#pragma unroll
+      for (int s = 0; s < NR; s++) { rows_v[s] = 0; rows_k[s] = 0; rows_n[s] = 0; raw[s] = 0; }
+      prefetch_raw(0, raw);
+      finish_rows(0, raw, rows0, nv_unused);
+      if (T > 1) { prefetch_raw(1, raw); finish_rows(1, raw, rows_v, nv_unused); }
+      if (T > 2) { prefetch_raw(2, raw); finish_rows(2, raw, rows_k, nv_unused); }
+      if (T > 3) prefetch_raw(3, raw);
+      issue(krsrc, k_srb, false, rows0, lds0);
+      issue(vrsrc, v_srb, true, rows0, lds0 + 2 * TILE);
+      if (T > 1) issue(krsrc, k_srb, false, rows_v, lds0 + TILE);
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      __syncthreads();   // the computing waves have read K(0): its buffer may be refilled
+      for (int t = 0; t + 1 < T; t++) {
+        const int par = t & 1;
+        issue(vrsrc, v_srb, true, rows_v, lds0 + (3 - par) * TILE);
+        if (t + 2 < T) issue(krsrc, k_srb, false, rows_k, lds0 + par * TILE);
+        if (t + 3 < T) finish_rows(t + 3, raw, rows_n, nv_unused);
+        if (t + 4 < T) prefetch_raw(t + 4, raw);
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < NR; s++) { rows_v[s] = rows_k[s]; rows_k[s] = rows_n[s]; }
+      }
+      __syncthreads();   // the one after the last tile
+      return;
+    }
 
     // Q^T fragments stay in registers for the whole key loop
     const int qrow = min(q0 + wave * 32 + r, p.Lq - 1);
@@ -330,7 +374,9 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
 #pragma unroll
     for (int s = 0; s < NR; s++) { rows_v[s] = 0; rows_k[s] = 0; rows_n[s] = 0; raw[s] = 0; }
     int nv0, nv1 = 64, nv2 = 64, nv3 = 64;
-    {
+    if (NPROD) {
+      nv0 = nvalid_gather(0); nv1 = nvalid_gather(1); nv2 = nvalid_gather(2);
+    } else {
       int rows0[NR];
       // tiles 0..3: block lists use the entries read next to the count
       auto first_raw = [&](int t, int (&raw)[NR]) {
@@ -354,6 +400,9 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     __syncthreads();
     f32x16 sa0, sa1, sb0, sb1;
     qk_tile(smem, sa0, sa1);
+    // K(2) is fetched into the buffer of K(0) at the top of the first iteration: every wave must have read
+    // K(0) before any wave issues that fill
+    __syncthreads();
     if (nv0 < 64) mask_tile(sa0, sa1, nv0);
     rescale_check(max_tile(sa0, sa1));
 
@@ -367,10 +416,14 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     auto body = [&](int t, auto par, auto masked, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1) {
       constexpr int PAR = decltype(par)::value;
       constexpr bool MASKED = decltype(masked)::value;
-      if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows_v, lds0 + (3 - PAR) * TILE);
-      if (t + 2 < T) issue(krsrc, k_srb, false, rows_k, lds0 + PAR * TILE);
-      if (t + 3 < T) finish_rows(t + 3, raw, rows_n, nv3);
-      if (t + 4 < T) prefetch_raw(t + 4, raw);
+      if (NPROD) {
+        nv3 = nvalid_gather(t + 3);
+      } else {
+        if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows_v, lds0 + (3 - PAR) * TILE);
+        if (t + 2 < T) issue(krsrc, k_srb, false, rows_k, lds0 + PAR * TILE);
+        if (t + 3 < T) finish_rows(t + 3, raw, rows_n, nv3);
+        if (t + 4 < T) prefetch_raw(t + 4, raw);
+      }
       // The block below is software-pipelined by hand; sched_barrier(0) after every step stops the
       // compiler from regrouping it.  Phase A: QK MFMA j | K-fragment read j+4 | softmax slot j of
       // S(t).  Phase B: PV MFMA j | the two transposing V reads of MFMA j+4 | the last softmax slots
@@ -477,8 +530,10 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       __syncthreads();
       rescale_check(mx);
       nv0 = nv1; nv1 = nv2; nv2 = nv3;
+      if (!NPROD) {
 #pragma unroll
-      for (int s = 0; s < NR; s++) { rows_v[s] = rows_k[s]; rows_k[s] = rows_n[s]; }
+        for (int s = 0; s < NR; s++) { rows_v[s] = rows_k[s]; rows_k[s] = rows_n[s]; }
+      }
     };
     auto step = [&](int t, auto par, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1) {
       if (nv1 < 64) body(t, par, std::true_type{}, c0, c1, n0, n1);
@@ -509,6 +564,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   }
 
   // ---- epilogue ----
+  if (NPROD && wave >= NCOMP) return;   // fetch waves own no query rows (only reached with an empty list)
   const float ltot = xhalf_sum(lsum);
   const bool empty = !(ltot > 0.f);
   const float inv = empty ? 0.f : 1.0f / ltot;
@@ -593,7 +649,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
 template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY>
 static int launch_one(const AttnParams& p0, hipStream_t stream) {
   AttnParams p = p0;
-  constexpr int WGROWS = NWAVES * 32;
+  constexpr int WGROWS = ((MODE == MODE_GATHER && NWAVES == 8) ? 6 : NWAVES) * 32;   // two of eight token-list waves only fetch
   constexpr int SMEM = 4 * 64 * D * 2;
   if (MODE == MODE_BLOCK && p.list == nullptr) p.group_rows = WGROWS;  // dense: any row grouping
   if (p.group_rows % WGROWS != 0) return LVAR_EINVAL;
@@ -612,6 +668,7 @@ static int launch_d(const AttnParams& p, int mode, bool accum, bool lse_only, in
   if (mode == MODE_BLOCK) {
     return lse_only ? launch_one<D, 4, MODE_BLOCK, false, true>(p, s) : launch_one<D, 4, MODE_BLOCK, false, false>(p, s);
   } else if (mode == MODE_GATHER) {
+    if (nwaves == 8) return launch_one<D, 8, MODE_GATHER, true, false>(p, s);
     if (nwaves == 6) return launch_one<D, 6, MODE_GATHER, true, false>(p, s);
     if (nwaves == 3) return launch_one<D, 3, MODE_GATHER, true, false>(p, s);
     if (nwaves == 2) return launch_one<D, 2, MODE_GATHER, true, false>(p, s);

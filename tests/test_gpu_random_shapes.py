@@ -116,3 +116,34 @@ def test_token_lists_slice_matches_full_launch():
         assert torch.equal(small, big[sl]), (b, h)
         ref = oracle.csp_attn(q[sl], k[sl], v[sl], None, idx[sl], counts[sl], o0[sl], 1)
         assert close(big[sl], ref), (b, h)
+
+
+def test_token_lists_fetch_waves_match_six_wave_groups(tmp_path):
+    """A 192-row group runs with six computing waves plus two fetch waves by default and with six waves that do
+    both under LVAR_CSP_WAVES=6 (read once per process, hence the child processes): same arithmetic per row,
+    so the outputs must agree bit for bit."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys, torch\n"
+        f"sys.path.insert(0, {root!r}); sys.path.insert(0, {os.path.join(root, 'tests')!r})\n"
+        "from conftest import make_qkv\n"
+        "from lvar_amd import sparse_attn_ops as ops\n"
+        "g = torch.Generator().manual_seed(11)\n"
+        "B, H, Lq, Lk, d = 1, 3, 500, 700, 128\n"
+        "q, k, v = make_qkv(B, H, Lq, Lk, d, seed=11, amp=0.5)\n"
+        "G = (Lq + 191) // 192\n"
+        "idx = torch.randint(0, Lk, (B, H, G, Lk), generator=g, dtype=torch.int32)\n"
+        "cnt = torch.randint(0, Lk + 1, (B, H, G), generator=g, dtype=torch.int32)\n"
+        "o0 = (torch.randn(B, H, Lq, d, generator=g) * 0.5).to(torch.bfloat16)\n"
+        "out = ops.csp_attn(q.cuda(), k.cuda(), v.cuda(), None, idx.cuda(), cnt.cuda(), o0.cuda(), -1)\n"
+        "torch.save(out.cpu(), sys.argv[1])\n")
+    outs = []
+    for waves in ("8", "6"):
+        path = str(tmp_path / f"o{waves}.pt")
+        env = dict(os.environ, LVAR_CSP_WAVES=waves)
+        subprocess.run([sys.executable, "-c", code, path], check=True, env=env, timeout=100)
+        outs.append(torch.load(path, weights_only=True))
+    assert torch.equal(outs[0], outs[1])
