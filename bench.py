@@ -37,7 +37,7 @@ MEASURED_TRAFFIC = {
     "dense": 240.8e6,
     # profiles/colsum_infinity2b_1024_last_scale.txt: FETCH 65760 KiB x 2.0 + WRITE 28990 KiB x 1.0
     "colsum": 164.4e6,
-    # profiles/attn_fwd_token_list_infinity2b_1024_last_scale_top20pct.txt: FETCH 141250 KiB x 2.0 + WRITE 32716 KiB x 1.0
+    # profiles/attn_fwd_token_list_infinity2b_1024_last_scale_top20pct.txt: FETCH 141270 KiB x 2.0 + WRITE 32717 KiB x 1.0
     "csp": 322.8e6,
 }
 
