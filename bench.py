@@ -407,13 +407,7 @@ def main():
         elif wl == "video_10":
             # 3D local window over a latent grid of 8 frames x 64 x 64 tokens (+-1 frame, +-1 spatial
             # block of 128 tokens) plus colsum top-k blocks (scores from every 4th query row) up to 10 % density
-            blk = torch.arange(nQ, device=dev)
-            f, s_ = blk // 32, blk % 32                                     # 32 blocks of 128 tokens per frame
-            near = ((f[:, None] - f[None, :]).abs() <= 1) & ((s_[:, None] - s_[None, :]).abs() <= 1)
-            cs = ops.colsum(qg[:, :, ::4].contiguous(), kg, scale, q_group_size=32)   # every 4th query row: 32 samples per 128-row block
-            score = mb.key_block_sums(cs, bk)[:, :, :nQ].contiguous()
-            del cs
-            num, idx = ops.block_topk_lists(score, int(round(0.10 * nK)), near)
+            num, idx, _ = mb.video_window_topk_block_lists(qg, kg, scale, density=0.10)
             mask = None
             config.update({"block": [bq, bk], "mask": "3D window (+-1 frame, +-1 spatial block) + colsum top-k blocks up to 10 %"})
         else:

@@ -21,6 +21,7 @@ __all__ = [
     "INFINITY_SCALES", "scale_offsets", "indices_count", "topk_index_list", "map_inds_counts_across_scales",
     "local_group_runs", "append_local_run", "upsample_ocache", "flex_block_mask", "block_mask_to_lists",
     "key_block_sums", "topk_block_lists", "sink_window_base_mask", "sink_window_topk_block_mask",
+    "video_window_base_mask", "video_window_topk_block_lists",
 ]
 
 
@@ -270,3 +271,42 @@ def sink_window_topk_block_mask(block_scores: torch.Tensor, block_q: int = 128, 
     score = block_scores.to(torch.float32).masked_fill(base, -float("inf"))
     rank = torch.argsort(torch.argsort(score, dim=-1, descending=True, stable=True), dim=-1, stable=True)
     return base | (rank < extra[None, None, :, None])
+
+
+def video_window_base_mask(frames: int = 8, height: int = 64, width: int = 64, block: int = 128, frame_radius: int = 1,
+                           spatial_radius: int = 1, device=None) -> torch.Tensor:
+    """3D local-window block mask for video tokens laid out frame by frame (``frames x height x width``,
+    row-major inside a frame), bool [nQ, nK] for ``block x block`` blocks: a key block is kept when it holds
+    a token whose frame is within ``frame_radius`` frames and whose spatial block (``block`` consecutive
+    tokens of a frame) is within ``spatial_radius`` of those of a token of the query block.  The frame length
+    must be a multiple of ``block`` (every block then lies in one frame and is one spatial block)."""
+    per_frame = height * width
+    if per_frame % block:
+        raise ValueError(f"tokens per frame ({per_frame}) must be a multiple of the block size ({block})")
+    bpf = per_frame // block
+    blk = torch.arange(frames * bpf, device=device)
+    f, s = blk // bpf, blk % bpf
+    return ((f[:, None] - f[None, :]).abs() <= frame_radius) & ((s[:, None] - s[None, :]).abs() <= spatial_radius)
+
+
+def video_window_topk_block_lists(q: torch.Tensor, k: torch.Tensor, scale=None, density: float = 0.10, frames: int = 8,
+                                  height: int = 64, width: int = 64, block: int = 128, query_stride: int = 4
+                                  ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Block lists of the long-video configuration: :func:`video_window_base_mask` plus the best-scoring
+    other key blocks per query block up to ``round(density * nK)`` blocks per row.  The scores are column
+    sums of the softmax probabilities of every ``query_stride``-th query row, summed per key block (the
+    colsum kernel and the block top-k kernel of the HIP library; ties go to the smaller block).  Returns
+    ``(kv_num_blocks [B,H,nQ], kv_indices [B,H,nQ,nK], block_scores [B,H,nQ,nK])``."""
+    from . import sparse_attn_ops as ops
+    Lq, Lk = q.shape[2], k.shape[2]
+    if Lq != frames * height * width or Lk != Lq:
+        raise ValueError(f"expected Lq = Lk = {frames * height * width}, got {Lq}, {Lk}")
+    if block % query_stride or (block // query_stride) % 32:
+        raise ValueError("block / query_stride must be a multiple of 32 (the colsum group size)")
+    nK = (Lk + block - 1) // block
+    base = video_window_base_mask(frames, height, width, block, device=q.device)
+    cs = ops.colsum(q[:, :, ::query_stride].contiguous(), k, scale, q_group_size=block // query_stride)
+    score = key_block_sums(cs, block).contiguous()
+    del cs
+    num, idx = ops.block_topk_lists(score, int(round(density * nK)), base)
+    return num, idx, score

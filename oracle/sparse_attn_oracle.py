@@ -29,6 +29,7 @@ __all__ = [
     "aggregate_group_indices", "upsample_ocache", "flex_block_mask", "infinity_cum",
     "INFINITY_SCALES", "config2_block_mask", "attn_flops_blocks", "attn_flops_lists",
     "topk_token_set", "append_local_run", "mask_to_lists", "window_key_scores",
+    "video_window_block_mask", "base_plus_topk_block_mask",
 ]
 
 # Infinity "1M" scale schedule, reference utils/dynamic_resolution.py:7 and
@@ -503,3 +504,46 @@ def attn_flops_lists(counts, Lq, d, bm=192):
     B, H, G = counts.shape
     rows = torch.tensor([min(bm, Lq - g * bm) for g in range(G)], dtype=torch.int64)
     return int(4 * d * (counts.long() * rows.view(1, 1, G)).sum().item())
+
+
+def video_window_block_mask(frames=8, height=64, width=64, block=128, frame_radius=1, spatial_radius=1):
+    """3D local-window block mask of the long-video benchmark configuration (no reference counterpart:
+    the configuration is defined by the benchmark, tokens laid out frame by frame), by brute force over
+    token pairs of every block pair: token t has frame ``t // (height*width)`` and spatial block
+    ``(t % (height*width)) // block``; a block pair is kept if ANY of its token pairs is within
+    ``frame_radius`` frames and ``spatial_radius`` spatial blocks.  bool [nQ, nK]."""
+    per = height * width
+    n = frames * per
+    nb = (n + block - 1) // block
+    tok = np.arange(n)
+    fr, sb = tok // per, (tok % per) // block
+    mask = np.zeros((nb, nb), dtype=bool)
+    for i in range(nb):
+        fi, si = fr[i * block:(i + 1) * block], sb[i * block:(i + 1) * block]
+        for j in range(nb):
+            fj, sj = fr[j * block:(j + 1) * block], sb[j * block:(j + 1) * block]
+            # token pairs of the two blocks: distinct (frame, spatial block) combinations are enough
+            pi = set(zip(fi.tolist(), si.tolist()))
+            pj = set(zip(fj.tolist(), sj.tolist()))
+            mask[i, j] = any(abs(a - c) <= frame_radius and abs(b - d_) <= spatial_radius for a, b in pi for c, d_ in pj)
+    return torch.from_numpy(mask)
+
+
+def base_plus_topk_block_mask(block_scores, base, target):
+    """``base`` [nQ,nK] (always kept) plus, per row, the best-scoring other blocks until ``target`` blocks
+    are kept; equal scores go to the smaller block index (the first entries of a stable descending sort).
+    block_scores [B,H,nQ,nK] -> bool [B,H,nQ,nK]."""
+    sc = np.asarray(block_scores.detach().to(torch.float32).cpu().numpy()).copy()
+    bs = np.asarray(base.cpu().numpy()).astype(bool)
+    B, H, nQ, nK = sc.shape
+    out = np.broadcast_to(bs, sc.shape).copy()
+    for i in range(nQ):
+        extra = max(0, target - int(bs[i].sum()))
+        if extra == 0:
+            continue
+        cand = np.where(~bs[i])[0]
+        for b in range(B):
+            for h in range(H):
+                order = cand[np.argsort(-sc[b, h, i, cand], kind="stable")]
+                out[b, h, i, order[:extra]] = True
+    return torch.from_numpy(out)

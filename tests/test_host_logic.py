@@ -120,3 +120,27 @@ def test_sink_window_topk_mask_matches_oracle():
         assert torch.equal(a, b)
     a = mb.sink_window_topk_block_mask(scores)
     assert bool((a.sum(-1) == 41).all())
+
+
+def test_flex_block_mask_hand_computed_fine_entries():
+    from test_oracle import check_flex_fine_cases
+    check_flex_fine_cases(mb.flex_block_mask)
+
+
+def test_video_window_base_mask_matches_oracle():
+    assert torch.equal(mb.video_window_base_mask(), oracle.video_window_block_mask())
+    for (f, h, w, blk, fr, sr) in ((3, 4, 8, 8, 1, 1), (4, 4, 4, 16, 1, 0), (2, 8, 8, 16, 0, 2), (5, 2, 8, 4, 2, 1)):
+        assert torch.equal(mb.video_window_base_mask(f, h, w, blk, fr, sr), oracle.video_window_block_mask(f, h, w, blk, fr, sr))
+    with pytest.raises(ValueError):
+        mb.video_window_base_mask(2, 2, 3, 4)
+
+
+def test_base_plus_topk_block_mask_equals_config2_selection():
+    g = torch.Generator().manual_seed(3)
+    scores = torch.rand(1, 2, 32, 165, generator=g)
+    scores[0, 0, 4, 100:120] = 0.5                                  # ties through the cut go to the smaller block
+    base = mb.sink_window_base_mask(128, 64)
+    want = oracle.config2_block_mask(scores)
+    got = oracle.base_plus_topk_block_mask(scores, base, round(0.25 * 165))
+    assert torch.equal(got, want)
+    assert torch.equal(mb.sink_window_topk_block_mask(scores), got)

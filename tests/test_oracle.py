@@ -231,6 +231,70 @@ def test_flex_block_mask_properties():
     assert torch.equal(pad.view(pad.shape[0], -1, 2).any(-1), m)
 
 
+# Hand-computed fine-grained entries (block_size = block_k = 1) of the sink + window predicate
+# (models/sparvar/basic_sparvar.py:113-151) on the schedule 2x2, 6x6, 4x4 with the 4x4 scale as queries:
+# key offsets cum = [0, 4, 40, 56]; kernel sizes per KEY scale [1, 3, 5] (half = 0, 1, 2).
+# Entry: (query (y, x), key scale, key (y, x), expected).
+FLEX_FINE_SCALES, FLEX_FINE_KERNELS, FLEX_FINE_CUM = [2, 6, 4], [1, 3, 5], [0, 4, 40, 56]
+FLEX_FINE_CASES = [
+    # rounding tie 1/4*2 = 0.5 -> 0 (half-to-even; half-up would give 1)
+    ((1, 0), 0, (0, 0), True), ((1, 0), 0, (1, 0), False),
+    # rounding tie 3/4*2 = 1.5 -> 2: the centre falls off the 2x2 grid, nothing of that scale is attended
+    ((3, 0), 0, (0, 0), False), ((3, 0), 0, (1, 0), False), ((3, 0), 0, (1, 1), False),
+    # rounding tie 3/4*6 = 4.5 -> 4 (half-to-even; half-up would give 5): rows 3..5 of the 6x6 scale
+    ((3, 0), 1, (3, 0), True), ((3, 0), 1, (5, 0), True),
+    # window edge, key-scale kernel 3: distance 1 = half is kept, distance 2 = half + 1 is not
+    # (the query scale's own kernel, 5, would keep distance 2)
+    ((3, 0), 1, (2, 0), False), ((3, 0), 1, (4, 1), True), ((3, 0), 1, (4, 2), False),
+    # rounding tie 1/4*6 = 1.5 -> 2 (both rules agree): rows 1..3
+    ((1, 0), 1, (1, 0), True), ((1, 0), 1, (0, 0), False), ((1, 0), 1, (3, 0), True), ((1, 0), 1, (4, 0), False),
+    # the query scale itself, kernel 5: distance 2 kept, distance 3 not
+    ((0, 0), 2, (2, 2), True), ((0, 0), 2, (3, 0), False), ((0, 0), 2, (0, 3), False), ((3, 3), 2, (1, 1), True),
+    ((3, 3), 2, (0, 3), False),
+]
+
+
+def flex_fine_entry(mask_fn, qyx, si, kyx, kernels=FLEX_FINE_KERNELS, sink=0):
+    side_q, side_k = FLEX_FINE_SCALES[2], FLEX_FINE_SCALES[si]
+    m = mask_fn(2, kernels, sink, 1, scales=FLEX_FINE_SCALES, block_k=1)
+    assert tuple(m.shape) == (16, 56)
+    return bool(m[qyx[0] * side_q + qyx[1], FLEX_FINE_CUM[si] + kyx[0] * side_k + kyx[1]])
+
+
+def check_flex_fine_cases(mask_fn):
+    for qyx, si, kyx, want in FLEX_FINE_CASES:
+        assert flex_fine_entry(mask_fn, qyx, si, kyx) == want, (qyx, si, kyx, want)
+    # sink: every key below cum[1] = 4 is attended by every query, also where the window misses
+    assert flex_fine_entry(mask_fn, (3, 0), 0, (0, 0), sink=1) and flex_fine_entry(mask_fn, (3, 0), 0, (1, 1), sink=1)
+    assert not flex_fine_entry(mask_fn, (3, 0), 1, (2, 0), sink=1)
+    # negative kernel size: -1 // 2 = -1, not even the centre key is attended
+    assert not flex_fine_entry(mask_fn, (1, 0), 1, (2, 0), kernels=[1, -1, 5])
+    assert flex_fine_entry(mask_fn, (1, 0), 1, (2, 0), kernels=[1, 1, 5])
+    # kernel 1 keeps the centre only
+    assert not flex_fine_entry(mask_fn, (1, 0), 1, (1, 0), kernels=[1, 1, 5])
+
+
+def test_flex_block_mask_hand_computed_fine_entries():
+    check_flex_fine_cases(oracle.flex_block_mask)
+
+
+def test_video_window_block_mask_hand_cases():
+    """8 frames x 64 x 64 tokens, 128-token blocks: 32 blocks per frame, block = (frame, spatial block)."""
+    m = oracle.video_window_block_mask()
+    assert m.shape == (256, 256) and bool((m == m.T).all())
+    assert bool(m[0, 0]) and bool(m[0, 1]) and not bool(m[0, 2])           # same frame: +-1 spatial block
+    assert bool(m[0, 32]) and bool(m[0, 33]) and not bool(m[0, 34])        # next frame
+    assert not bool(m[0, 64]) and not bool(m[0, 31])                       # two frames away; far end of the frame
+    assert bool(m[40, 7]) and bool(m[40, 9]) and bool(m[40, 73]) and not bool(m[40, 104]) and not bool(m[40, 10])
+    assert int(m[0].sum()) == 4 and int(m[40].sum()) == 9 and int(m[255].sum()) == 4 and int(m[31].sum()) == 4
+    assert int(m[5].sum()) == 6 and int(m[32].sum()) == 6                  # frame edge / spatial edge
+    # a layout whose blocks straddle frames: 2 frames x 2 x 3 tokens, 4-token blocks
+    s = oracle.video_window_block_mask(2, 2, 3, 4, frame_radius=0, spatial_radius=0)
+    # tokens 0..5 are frame 0 (spatial blocks 0,0,0,0,1,1), tokens 6..11 frame 1 (same pattern); the blocks
+    # {0..3}, {4..7}, {8..11} hold the (frame, spatial block) pairs {(0,0)}, {(0,1),(1,0)}, {(1,0),(1,1)}
+    assert s.tolist() == [[True, False, False], [False, True, True], [False, True, True]]
+
+
 def test_config2_block_mask_density():
     scores = rnd(1, 2, 32, 165, seed=22).abs()
     mask = oracle.config2_block_mask(scores)
