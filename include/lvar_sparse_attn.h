@@ -22,7 +22,7 @@ extern "C" {
 
 #define LVAR_OK 0
 #define LVAR_EINVAL (-1)      /* bad size / null pointer / misaligned pointer or stride */
-#define LVAR_EUNSUPPORTED (-2) /* head_dim or block shape not built */
+#define LVAR_EUNSUPPORTED (-2) /* head_dim, block shape or query-group size not built */
 #define LVAR_ELAUNCH (-3)      /* HIP reported a launch error */
 
 /* Tensor view: base pointer plus element strides of a [B,H,rows,d] bf16 tensor (d stride 1). */
@@ -53,6 +53,16 @@ int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_
                         float scale, void* stream);
 
 /*
+ * Dense flash-attention forward returning the per-row constant of the reference's native op:
+ * rcp[b,h,i] = 1 / (2^M * L) (fp32 contiguous [B,H,Lq]), the `l_vec` that torch.ops.chipmunk.dense_attn
+ * returns beside o (kernels/chipmunk/csrc/attn/dense_attn.cu:227-230, schema at chipmunk.cu:57) and that
+ * torch.ops.chipmunk.dense_colsum_attn takes as its fourth argument.  o and rcp must not be NULL.
+ */
+int lvar_dense_attn_rcp_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* rcp,
+                            int B, int H, int Lq, int Lk, int head_dim,
+                            float scale, void* stream);
+
+/*
  * Colsum given the row statistics: cs[b,h,g,n] = sum_{i in group g} exp2(q_i.k_n*scale*log2e - lse2_i),
  * lse2 = M + log2(L) (fp32 contiguous [B,H,Lq], as written by lvar_dense_attn_fwd), groups of
  * q_group_size consecutive query rows (a multiple of 32), rows >= Lq add zero.
@@ -76,8 +86,11 @@ int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* 
  * [B,H,G,idx_row_stride] (row stride in elements, >= max count), counts int32 [B,H,G]
  * contiguous, clamped to [0, idx_row_stride].  Indices outside [0,Lk) are clamped.  count == 0 leaves o = o_accum,
  * M = -inf, L = 1.  o_accum may be NULL (treated as zero) and may alias o.
- * group_rows must be a multiple of 32 (the reference uses 192).  Gathered rows are addressed with a 24-bit
- * multiply: Lk <= 2^24 and K/V row strides below 2^23 elements, else LVAR_EUNSUPPORTED.
+ * group_rows (query rows sharing one list; the reference uses 192) must be a multiple of 64 or of 96, else
+ * LVAR_EUNSUPPORTED.  Gathered rows are addressed with a 24-bit multiply: Lk <= 2^24 and K/V row strides
+ * below 2^23 elements, else LVAR_EUNSUPPORTED.  A count that is not a multiple of 64 is honoured exactly:
+ * the last tile is masked at the count (the reference attends whole 64-entry tiles, attn_csp.py:53-70,
+ * and therefore requires counts that are multiples of 64).
  * Replaces sattn_triton.csp_attn (kernels/sparse_attn/triton/attn_csp.py:215-265) and
  * torch.ops.chipmunk.csp_attn (kernels/chipmunk/csrc/chipmunk.cu:59,
  * kernels/chipmunk/csrc/attn/csp_attn.cu:318-433).
@@ -181,8 +194,11 @@ int lvar_remap_concat_lists(const int32_t* src_indices, int64_t src_row_stride, 
  * ascending columns of its non-zero entries to indices[row, :] (row stride idx_row_stride >= n), round
  * the count up to a multiple of `multiple_of` (capped at n) by appending the lowest zero columns, zero
  * the rest of the n columns, and store the padded count in counts[row].  With multiple_of = 1 and a
- * block mask this yields flex BlockMask lists (kv_num_blocks / kv_indices).  Same result as the
- * reference's mask_to_indices (kernels/chipmunk/csrc/indexed_io/mask_to_indices.cu:21-97).
+ * block mask this yields flex BlockMask lists (kv_num_blocks / kv_indices).  Counterpart of the
+ * reference's mask_to_indices (kernels/chipmunk/csrc/indexed_io/mask_to_indices.cu:21-97) with two
+ * stated differences: the list is in ascending column order (the reference writes a thread-strided order;
+ * the SET is the same), and the padded count is capped at n (the reference's rounded count can exceed the
+ * row, mask_to_indices.cu:62,93).
  */
 int lvar_mask_to_lists(const uint8_t* mask, int64_t mask_row_stride,
                        int32_t* indices, int64_t idx_row_stride, int32_t* counts,

@@ -12,7 +12,7 @@ from .build import LIB_PATH
 
 EXPORTED_SYMBOLS = (
     "lvar_version", "lvar_target_arch", "lvar_status_string",
-    "lvar_dense_attn_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_csp_attn_upsample_fwd",
+    "lvar_dense_attn_fwd", "lvar_dense_attn_rcp_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_csp_attn_upsample_fwd",
     "lvar_block_sparse_attn_fwd",
     "lvar_block_topk_lists", "lvar_topk_token_lists", "lvar_remap_concat_lists", "lvar_mask_to_lists",
     "lvar_window_key_scores",
@@ -51,6 +51,8 @@ def load() -> C.CDLL:
     lib.lvar_status_string.argtypes = [I]
     lib.lvar_dense_attn_fwd.restype = I
     lib.lvar_dense_attn_fwd.argtypes = [T, T, T, T, P, P, P, I, I, I, I, I, F, P]
+    lib.lvar_dense_attn_rcp_fwd.restype = I
+    lib.lvar_dense_attn_rcp_fwd.argtypes = [T, T, T, T, P, I, I, I, I, I, F, P]
     lib.lvar_colsum_fwd.restype = I
     lib.lvar_colsum_fwd.argtypes = [T, T, P, P, P, I, I, I, I, I, I, F, P]
     lib.lvar_csp_attn_fwd.restype = I
@@ -98,9 +100,13 @@ def torch_binding():
         spec = importlib.util.spec_from_file_location("_lvar_torch", path)
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
-        mod.bind(C.cast(load().lvar_dense_attn_fwd, C.c_void_p).value)
+        lib = load()
+        mod.bind(C.cast(lib.lvar_dense_attn_fwd, C.c_void_p).value, C.cast(lib.lvar_dense_attn_rcp_fwd, C.c_void_p).value)
         _binding = mod
-    except Exception:          # a stale or incompatible module must not take the ctypes path down with it
+    except Exception as e:     # a stale or incompatible module must not take the ctypes path down with it
+        import warnings
+        warnings.warn(f"lvar_amd: the compiled torch binding {path} did not load ({type(e).__name__}: {e}); "
+                      "dense_attn runs through the slower ctypes path.  Rebuild it with `python -m lvar_amd.build`.",
+                      RuntimeWarning, stacklevel=2)
         _binding = None
     return _binding
-

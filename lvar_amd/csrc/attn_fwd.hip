@@ -3,7 +3,7 @@
 //
 // Work decomposition
 //   workgroup  = NWAVES waves, 32 query rows per wave, all waves share the K/V tiles in LDS
-//                (token lists: 8 waves = 6 computing waves + 2 waves that only fetch, see NPROD)
+//                (token lists with 192-row groups: 8 waves = 6 computing waves + 2 waves that only fetch, see NPROD)
 //   wave       = S^T[64 keys x 32 queries] = K_tile . Q^T with 32x32x16 bf16 MFMA (K rows are
 //                the A operand read from LDS, Q^T is the B operand held in registers), so a
 //                lane owns ONE query column: the softmax row max / sum are in-register
@@ -40,7 +40,7 @@ namespace lvar {
 template <int NQK, int HB, int EA>
 struct ExpSlots {
   static constexpr int lo(int g) {
-    return g <= 0 ? 0 : g < NQK ? g * EA / NQK : g < NQK + HB ? EA + (g - NQK) * (32 - EA) / HB : 32;
+    return g <= 0 ? 0 : g < NQK ? g * EA / NQK : g < NQK + HB ? EA + (g - NQK) * (32 - EA) / (HB ? HB : 1) : 32;
   }
 };
 
@@ -137,16 +137,18 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const float c = p.c;
 
   if (T > 0) {
-    // raw buffer descriptors of this (batch, head) slice of K and V: base, stride 0, no bound
-    auto make_rsrc = [](const void* base) -> i32x4 {
+    // raw buffer descriptors of this (batch, head) slice of K and V: base, stride 0, bound = the bytes of
+    // the slice (below 2^31, checked on the host), so a fill beyond the last key row reads zeros
+    auto make_rsrc = [](const void* base, int bytes) -> i32x4 {
       const uint64_t a = (uint64_t)base;
       i32x4 rs = {__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
-                  __builtin_amdgcn_readfirstlane((int)(uint32_t)((a >> 32) & 0xffffu)), 0x7fffffff, 0x00020000};
+                  __builtin_amdgcn_readfirstlane((int)(uint32_t)((a >> 32) & 0xffffu)),
+                  __builtin_amdgcn_readfirstlane(bytes), 0x00020000};
       return rs;
     };
-    const i32x4 krsrc = make_rsrc(p.k + b * p.k_sb + h * p.k_sh);
-    const i32x4 vrsrc = make_rsrc(p.v + b * p.v_sb + h * p.v_sh);
     const int k_srb = (int)p.k_sr * 2, v_srb = (int)p.v_sr * 2;  // row strides in bytes
+    const i32x4 krsrc = make_rsrc(p.k + b * p.k_sb + h * p.k_sh, (p.Lk - 1) * k_srb + ROWB);
+    const i32x4 vrsrc = make_rsrc(p.v + b * p.v_sb + h * p.v_sh, (p.Lk - 1) * v_srb + ROWB);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(LVAR_LDS char*)smem;
 
     // per-lane role in a tile load: row (within the RPI rows of one instruction) and chunk slot
@@ -172,7 +174,8 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     };
     auto finish_rows = [&](int t, const int (&raw)[NR], int (&rows)[NR], int& nvalid) {
       if (MODE == MODE_BLOCK) {
-        const int blk = __builtin_amdgcn_readfirstlane(raw[0]);
+        // a block index outside the key range (a caller's mistake) is clamped before it is scaled
+        const int blk = max(0, min(__builtin_amdgcn_readfirstlane(raw[0]), (p.Lk - 1) >> (6 + sub_shift)));
         rows[0] = ((blk << sub_shift) + (t & ((1 << sub_shift) - 1))) << 6;
         nvalid = max(0, min(64, p.Lk - rows[0]));
       } else {
@@ -574,6 +577,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     if (p.M) p.M[off] = empty ? -INFINITY : m_true;
     if (p.L) p.L[off] = empty ? 1.0f : ltot * fast_exp2(m_ref - m_true);
     if (p.LSE2) p.LSE2[off] = empty ? -INFINITY : m_ref + __builtin_amdgcn_logf(ltot);
+    if (p.RCP) p.RCP[off] = empty ? INFINITY : fast_exp2(-m_ref) * inv;
   }
   if (LSE_ONLY) return;
 
@@ -669,7 +673,6 @@ static int launch_d(const AttnParams& p, int mode, bool accum, bool lse_only, in
     return lse_only ? launch_one<D, 4, MODE_BLOCK, false, true>(p, s) : launch_one<D, 4, MODE_BLOCK, false, false>(p, s);
   } else if (mode == MODE_GATHER) {
     if (nwaves == 8) return launch_one<D, 8, MODE_GATHER, true, false>(p, s);
-    if (nwaves == 6) return launch_one<D, 6, MODE_GATHER, true, false>(p, s);
     if (nwaves == 3) return launch_one<D, 3, MODE_GATHER, true, false>(p, s);
     if (nwaves == 2) return launch_one<D, 2, MODE_GATHER, true, false>(p, s);
   }

@@ -1,7 +1,6 @@
 // extern "C" entry points declared in include/lvar_sparse_attn.h: argument validation and
 // parameter packing; all device work is in attn_fwd.hip / colsum.hip.
 #include <cmath>
-#include <cstdlib>
 #include "../../include/lvar_sparse_attn.h"
 #include "launch.h"
 
@@ -27,18 +26,16 @@ bool shape_ok(int B, int H, int Lq, int Lk, float scale) {
   return B > 0 && H > 0 && Lq > 0 && Lk > 0 && std::isfinite(scale) && scale > 0.f;
 }
 
-// Waves per workgroup of the token-list kernel.  A 192-row group runs as one 8-wave workgroup per CU: six
-// computing waves and two waves that only read the list and issue the K/V fills (they take the two wave
-// slots that six 256-register waves leave free).  Six waves that do both are ~6 % slower; two 3-wave
-// workgroups per group double the fills and spill registers, and are only taken when the group size is not a
-// multiple of 192 rows.  LVAR_CSP_WAVES=2|3|6|8 overrides the first choice.
-int gather_waves() {
-  static int v = [] {
-    const char* e = std::getenv("LVAR_CSP_WAVES");
-    const int n = e ? std::atoi(e) : 8;
-    return (n == 2 || n == 3 || n == 6 || n == 8) ? n : 8;
-  }();
-  return v;
+// Waves per workgroup of the token-list kernel, by the number of query rows that share a list.  A multiple
+// of 192 rows (the reference's group size) runs as one 8-wave workgroup per 192 rows: six computing waves
+// and two waves that only read the list and issue the K/V fills (they take the two wave slots that six
+// 256-register waves leave free on a CU).  Other multiples of 96 or 64 rows run as 3- or 2-wave workgroups
+// that each fetch for themselves.  0 = unsupported group size.
+int gather_waves(int group_rows) {
+  if (group_rows % 192 == 0) return 8;
+  if (group_rows % 96 == 0) return 3;
+  if (group_rows % 64 == 0) return 2;
+  return 0;
 }
 
 void fill_qkv(AttnParams& p, const lvar_tensor_t& q, const lvar_tensor_t& k, const lvar_tensor_t& v) {
@@ -58,27 +55,38 @@ const char* lvar_status_string(int status) {
   switch (status) {
     case LVAR_OK: return "ok";
     case LVAR_EINVAL: return "invalid argument (size, null/misaligned pointer, stride or scale)";
-    case LVAR_EUNSUPPORTED: return "unsupported head_dim or block shape";
+    case LVAR_EUNSUPPORTED: return "unsupported head_dim, block shape or query-group size";
     case LVAR_ELAUNCH: return "HIP launch failed";
     default: return "unknown status";
   }
 }
 
-int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
-                        float* LSE2, int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
+static int dense_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+                        float* LSE2, float* RCP, int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k)) return LVAR_EINVAL;
   const bool lse_only = (o.ptr == nullptr);
   if (!kv_span_ok(k, Lk, head_dim) || (!lse_only && !kv_span_ok(v, Lk, head_dim))) return LVAR_EINVAL;
-  if (!lse_only && (!view_ok(v) || !view_ok(o))) return LVAR_EINVAL;
-  if (lse_only && !((M && L) || LSE2)) return LVAR_EINVAL;
+  if (!lse_only && (!view_ok(v) || !view_ok(o) || o.stride_row <= 0)) return LVAR_EINVAL;
+  if (lse_only && !((M && L) || LSE2 || RCP)) return LVAR_EINVAL;
   AttnParams p{};
   fill_qkv(p, q, k, lse_only ? k : v);
   p.o = (bf16_t*)o.ptr; p.o_sb = o.stride_b; p.o_sh = o.stride_h; p.o_sr = o.stride_row;
-  p.M = M; p.L = L; p.LSE2 = LSE2;
+  p.M = M; p.L = L; p.LSE2 = LSE2; p.RCP = RCP;
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
   p.c = scale * kLog2e; p.o_scale = 1.f;
   p.list = nullptr; p.cnt = nullptr; p.group_rows = 128; p.sub_shift = 0;
   return launch_attn(p, head_dim, MODE_BLOCK, false, lse_only, 4, (hipStream_t)stream);
+}
+
+int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+                        float* LSE2, int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
+  return dense_common(q, k, v, o, M, L, LSE2, nullptr, B, H, Lq, Lk, head_dim, scale, stream);
+}
+
+int lvar_dense_attn_rcp_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* rcp,
+                            int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
+  if (!o.ptr || !rcp) return LVAR_EINVAL;
+  return dense_common(q, k, v, o, nullptr, nullptr, nullptr, rcp, B, H, Lq, Lk, head_dim, scale, stream);
 }
 
 int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* cs, float* block_sums,
@@ -102,12 +110,12 @@ static int csp_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_te
                       int64_t idx_row_stride, int group_rows, int B, int H, int Lq, int Lk, int head_dim,
                       float o_scale, float scale, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
-  if (o_accum.ptr && !view_ok(o_accum)) return LVAR_EINVAL;
+  if (o.stride_row <= 0 || (o_accum.ptr && (!view_ok(o_accum) || o_accum.stride_row <= 0))) return LVAR_EINVAL;
   if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
   // gathered rows are addressed with a 24-bit multiply: token index and row stride in bytes below 2^24
   if (Lk > (1 << 24) || k.stride_row * 2 >= (1 << 24) || v.stride_row * 2 >= (1 << 24)) return LVAR_EUNSUPPORTED;
   if (!indices || !counts || G <= 0 || idx_row_stride <= 0) return LVAR_EINVAL;
-  if (group_rows <= 0 || group_rows % 32 != 0 || (int64_t)G * group_rows < Lq) return LVAR_EINVAL;
+  if (group_rows <= 0 || (int64_t)G * group_rows < Lq) return LVAR_EINVAL;
   AttnParams p{};
   fill_qkv(p, q, k, v);
   p.o = (bf16_t*)o.ptr; p.o_sb = o.stride_b; p.o_sh = o.stride_h; p.o_sr = o.stride_row;
@@ -121,12 +129,8 @@ static int csp_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_te
   p.list_len = (int)(idx_row_stride > 0x7fffffff ? 0x7fffffff : idx_row_stride);
   p.group_rows = group_rows;
   p.up_src = up_src; p.up_dst = up_dst;
-  int nw = gather_waves();
-  if (nw == 8 && group_rows % 192 != 0) nw = 6;     // 8 = six computing waves + two fetch waves
-  while (nw != 8 && group_rows % (nw * 32) != 0) nw = (nw == 6) ? 3 : (nw == 3 ? 2 : 1);
-  if (nw == 1) {
-    if (group_rows % 64 == 0) nw = 2; else return LVAR_EUNSUPPORTED;
-  }
+  const int nw = gather_waves(group_rows);
+  if (nw == 0) return LVAR_EUNSUPPORTED;
   return launch_attn(p, head_dim, MODE_GATHER, true, false, nw, (hipStream_t)stream);
 }
 
@@ -157,7 +161,7 @@ int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
                                int head_dim, float scale, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
   if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
-  if (!kv_num_blocks || !kv_indices || nk_max <= 0) return LVAR_EINVAL;
+  if (!kv_num_blocks || !kv_indices || nk_max <= 0 || o.stride_row <= 0) return LVAR_EINVAL;
   if (block_q != 128 || (block_k != 64 && block_k != 128)) return LVAR_EUNSUPPORTED;
   AttnParams p{};
   fill_qkv(p, q, k, v);

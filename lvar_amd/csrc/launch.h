@@ -15,6 +15,7 @@ struct AttnParams {
   bf16_t* o;
   const bf16_t* o_accum;
   float *M, *L, *LSE2;
+  float* RCP;     // optional per-row constant 1 / (2^M * L)
   int64_t q_sb, q_sh, q_sr;
   int64_t k_sb, k_sh, k_sr;
   int64_t v_sb, v_sh, v_sr;

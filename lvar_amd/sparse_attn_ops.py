@@ -1,7 +1,8 @@
 """Operator API of the sparse-attention path, signature-compatible with the reference's
 ``kernels/sparse_attn/sparse_attn_ops.py`` (``dense_attn`` :21-59, ``dense_colsum_attn_s`` :65-113,
 ``dense_colsum_attn_q`` :119-149, ``csp_attn`` :273-292) and with the kernel-level functions of
-``kernels/sparse_attn/triton/__init__.py`` (``dense_colsum_attn``, ``csp_attn_delta``).
+``kernels/sparse_attn/triton/__init__.py`` (``dense_colsum_attn``, ``csp_attn_delta``; under the reference's own
+names in :mod:`lvar_amd.sattn_kernels`).
 
 Tensor contract: q ``[B,H,Lq,d]``, k/v ``[B,H,Lk,d]`` bf16 on a HIP device, unit stride on d;
 ``cs`` fp32 ``[B,H,ceil(Lq/bm),Lk]``; ``indices`` int32 ``[B,H,G,Lk]`` (valid prefix ``counts``),
@@ -128,7 +129,8 @@ def dense_attn(q, k, v, scale=None):
     Triton-provider return convention: ``lse`` is the tuple ``(M, L)``, each ``[B,H,Lq,1]``)."""
     fast = _lib.torch_binding()
     if fast is not None:
-        r = fast.fast_dense_attn(q, k, v, scale)      # None unless the inputs are the plain contiguous bf16 case
+        # None unless the inputs are the plain contiguous bf16 case
+        r = fast.fast_dense_attn(q, k, v, None if scale is None else float(scale)) if isinstance(q, torch.Tensor) else None
         if r is not None:
             return r[0], (r[1], r[2])
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
@@ -203,7 +205,7 @@ def dense_colsum_attn_q(q, k, v, scale=None):
     return dense_colsum_attn_s(q, k, v, scale)
 
 
-def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, upsample_from=None):
+def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, upsample_from=None, out=None):
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
     _check_qkv(q, k, v)
     B, H, Lq, d = q.shape
@@ -222,7 +224,8 @@ def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, u
         indices = indices.contiguous()
     counts = counts.contiguous()
     if o_accum is not None:
-        o_accum = _prep(o_accum, "o")
+        if o_accum is not out:
+            o_accum = _prep(o_accum, "o")
         if upsample_from is None:
             _require(o_accum.shape == q.shape, lambda: f"Output shape mismatch - o: {tuple(o_accum.shape)}, q: {tuple(q.shape)}")
         else:
@@ -230,7 +233,8 @@ def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, u
             _require(dst * dst == Lq and tuple(o_accum.shape) == (B, H, src * src, d),
                      lambda: f"O-cache shape mismatch - o_cache: {tuple(o_accum.shape)}, expected {(B, H, src * src, d)} "
                      f"for a {src}x{src} -> {dst}x{dst} grid, q: {tuple(q.shape)}")
-    o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device)
+    # `out` (the in-place op): the caller's tensor is the destination; it may alias o_accum
+    o = torch.empty((B, H, Lq, d), dtype=q.dtype, device=q.device) if out is None else out
     M = L = None
     if want_stats:
         M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
@@ -414,8 +418,10 @@ def mask_to_lists(mask, multiple_of: int = 1):
     """Compaction of a boolean mask ``[..., n]`` on the GPU: ``(counts int32 [...], indices int32 [..., n])``
     with the ascending set columns first, the count rounded up to ``multiple_of`` with the lowest unset
     columns as padding, and a zero tail.  For a block mask ``[B,H,nQ,nK]`` and ``multiple_of = 1`` these are
-    the flex ``BlockMask`` lists ``(kv_num_blocks, kv_indices)`` taken by :func:`block_sparse_attn`
-    (kernels/chipmunk/csrc/indexed_io/mask_to_indices.cu:21-97)."""
+    the flex ``BlockMask`` lists ``(kv_num_blocks, kv_indices)`` taken by :func:`block_sparse_attn`.
+    Counterpart of the reference's ``mask_to_indices`` (kernels/chipmunk/csrc/indexed_io/mask_to_indices.cu:21-97):
+    the same set, but in ascending order (the reference's order is thread-strided) and with the padded count
+    capped at ``n`` (the reference's rounded count can exceed the row)."""
     if not mask.is_cuda:
         raise RuntimeError("mask must live on a HIP device; lvar_amd has no CPU path")
     m = mask.to(torch.uint8).contiguous()

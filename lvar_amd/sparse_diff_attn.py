@@ -13,10 +13,21 @@ from . import sparse_attn_ops as ops
 from .sparse_attn_config import GLOBAL_CONFIG, get_kernel_config_attn
 
 
-class SparseDiffAttn:
-    def __init__(self, layer_num: int = 0, use_o_cache: bool = True, scales: Sequence[int] = mb.INFINITY_SCALES,
-                 spsd_scale: int = 10, speedup: bool = False):
+class SparseDiffAttn(torch.nn.Module):
+    """Constructor arguments as the reference's (models/sparvar/sparse_attn.py:866-873; constructed at
+    basic_sparvar.py:255-259 as ``SparseDiffAttn(layer_num, layer_counter, use_o_cache=True, spsd_scale=...)``).
+    ``layer_counter`` is any object with an ``increment()`` method (the reference's ``LayerCounter``) or None; it
+    is advanced once per call, as the reference does (sparse_attn.py:1151,1163).  ``wind_size`` is accepted and
+    unused: the reference overwrites it with ``GLOBAL_CONFIG['attn']['cs4a_ws']`` (sparse_attn.py:905-906)."""
+
+    def __init__(self, layer_num: int = 0, layer_counter=None, use_o_cache: bool = True,
+                 scales: Sequence[int] = mb.INFINITY_SCALES, spsd_scale: int = 10, wind_size: Optional[Sequence[int]] = None,
+                 speedup: bool = False):
+        super().__init__()
+        if isinstance(layer_counter, bool):
+            raise TypeError("the second argument is the layer counter (sparse_attn.py:867), not use_o_cache")
         self.layer_num = layer_num
+        self.layer_counter = layer_counter
         self.use_o_cache = use_o_cache
         self.scales = tuple(scales)
         self.spsd_scale = spsd_scale
@@ -38,6 +49,12 @@ class SparseDiffAttn:
         self.out_cache = None
 
     def forward(self, q, k, v, scale, do_full_step: bool = False, inference_step: int = 0, scale_ind: int = 0, layer_ind: int = 0):
+        out = self._fast_attention(q, k, v, scale, do_full_step, scale_ind)
+        if self.layer_counter is not None:
+            self.layer_counter.increment()
+        return out
+
+    def _fast_attention(self, q, k, v, scale, do_full_step: bool, scale_ind: int):
         if not GLOBAL_CONFIG["attn"]["is_enabled"]:
             return ops.dense_attn(q, k, v, scale)[0]
         top_keys = GLOBAL_CONFIG["attn"]["top_keys"]
@@ -76,4 +93,3 @@ class SparseDiffAttn:
             return ops.csp_attn_upsampled(q, k, v, scale, inds, counts, o, 1)
         return ops.csp_attn(q, k, v, scale, inds, counts, torch.zeros_like(q), 1)
 
-    __call__ = forward

@@ -1,14 +1,22 @@
-"""``torch.ops.lvar.*``: the three attention ops with the schemas the reference registers as
+"""Torch-library registration of the three attention ops with the schemas the reference registers as
 ``torch.ops.chipmunk.*`` (kernels/chipmunk/csrc/chipmunk.cu:57-59), for callers that use the
 torch-library entry points directly (``SelfAttention.forward`` calls ``torch.ops.chipmunk.dense_attn``,
 models/sparvar/basic_sparvar.py:384).  Like the reference's CUDA ops the softmax scale is fixed to 1
 (Infinity's cosine attention, dense_attn.cu:161-163); ``lse`` / ``p`` / ``l`` are the reference's
 per-row constant ``1 / (2^M * L)`` with the 1 = e^0 scale folded in, shape ``[B,H,Lq,1]``.
 
-    import lvar_amd.torch_ops          # registers the ops
+    import lvar_amd.torch_ops          # registers torch.ops.lvar.*
     o, lse = torch.ops.lvar.dense_attn(q, k, v)
     o, cs, l = torch.ops.lvar.dense_colsum_attn(q, k, v, lse)
     torch.ops.lvar.csp_attn(q, k, v, o, indices, counts, -1)      # in place on o
+
+    lvar_amd.torch_ops.register_as("chipmunk")    # opt-in: the reference's call sites then run unedited
+
+``dense_attn`` is implemented natively (checks, allocation and launch in C++, ``csrc/torch_binding.cpp``)
+when the compiled binding is built; the other two ops run at shapes where the kernel, not the host, is
+the bound and are Python implementations over the same C ABI.  Differences from the reference's CUDA ops:
+``cs`` is fp32 ``[B,H,ceil(Lq/192),Lk]`` without row padding (the reference returns bf16 with the row
+stride padded to a multiple of 8), and head_dim may be 64 as well as 128.
 """
 from __future__ import annotations
 
@@ -18,17 +26,25 @@ from . import _lib
 from . import sparse_attn_ops as ops
 from .sparse_attn_config import get_kernel_config_attn
 
-_lib_def = torch.library.Library("lvar", "DEF")
-_lib_def.define("csp_attn(Tensor q, Tensor k, Tensor v, Tensor(a!) o, Tensor indices, Tensor indices_counts, int o_scale) -> ()")
-_lib_def.define("dense_attn(Tensor q, Tensor k, Tensor v) -> Tensor[]")
-_lib_def.define("dense_colsum_attn(Tensor q, Tensor k, Tensor v, Tensor p) -> Tensor[]")
+_SCHEMAS = {
+    "csp_attn": "csp_attn(Tensor q, Tensor k, Tensor v, Tensor(a!) o, Tensor indices, Tensor indices_counts, int o_scale) -> ()",
+    "dense_attn": "dense_attn(Tensor q, Tensor k, Tensor v) -> Tensor[]",
+    "dense_colsum_attn": "dense_colsum_attn(Tensor q, Tensor k, Tensor v, Tensor p) -> Tensor[]",
+}
+_registered = {}      # namespace -> the torch.library.Library objects that keep the registration alive
 
 
 def _dense_attn(q, k, v):
     q, k, v = ops._prep(q, "q"), ops._prep(k, "k"), ops._prep(v, "v")
     ops._check_qkv(q, k, v)
-    o, _, _, lse2 = ops._dense_launch(q, k, v, 1.0, want_ml=False, want_lse2=True)
-    return [o, torch.exp2(-lse2).unsqueeze(-1)]
+    B, H, Lq, d = q.shape
+    o = torch.empty_like(q)
+    rcp = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
+    with ops._on_device(q):
+        st = _lib.load().lvar_dense_attn_rcp_fwd(ops._view(q), ops._view(k), ops._view(v), ops._view(o), rcp.data_ptr(),
+                                                B, H, Lq, k.shape[2], d, 1.0, ops._stream(q))
+    _lib.check(st, "lvar_dense_attn_rcp_fwd")
+    return [o, rcp]
 
 
 def _dense_colsum_attn(q, k, v, p):
@@ -45,23 +61,40 @@ def _dense_colsum_attn(q, k, v, p):
 def _csp_attn(q, k, v, o, indices, indices_counts, o_scale):
     if o_scale not in (1, -1):
         raise ValueError("o_scale must be 1 or -1")          # csp_attn.cu:330
-    qq, kk, vv = ops._prep(q, "q"), ops._prep(k, "k"), ops._prep(v, "v")
-    ops._check_qkv(qq, kk, vv)
-    if o.dtype != torch.bfloat16 or o.stride(-1) != 1 or tuple(o.shape) != tuple(q.shape):
-        raise ops.ShapeError("o must be a bf16 tensor shaped like q with unit stride on the head dimension")
-    B, H, Lq, d = qq.shape
-    G = indices.shape[2]
-    bm = get_kernel_config_attn()["bm"]
-    indices = indices.contiguous() if indices.stride(3) != 1 else indices
-    counts = indices_counts.contiguous()
-    with torch.cuda.device(qq.device):
-        st = _lib.load().lvar_csp_attn_fwd(ops._view(qq), ops._view(kk), ops._view(vv), ops._view(o), ops._view(o), None, None,
-                                          indices.data_ptr(), counts.data_ptr(), G, indices.stride(2), bm,
-                                          B, H, Lq, kk.shape[2], d, float(o_scale), 1.0, ops._stream(qq))
-    _lib.check(st, "lvar_csp_attn_fwd")
+    if o.dtype != torch.bfloat16 or o.stride(-1) != 1 or tuple(o.shape) != tuple(q.shape) or o.device != q.device \
+            or any(s % 8 for s in o.stride()[:-1]) or o.data_ptr() % 16:
+        raise ops.ShapeError("o must be a 16-byte aligned bf16 tensor shaped like q, on q's device, with unit stride on the "
+                             "head dimension and strides that are multiples of 8")
+    # same list checks as the operator-level csp_attn (dtype, dims, counts shape, device, packed (b,h,g) strides);
+    # the result is accumulated in place: o is both the addend and the destination
+    ops._csp_launch(q, k, v, indices, indices_counts, o, o_scale, 1.0, False, out=o)
 
 
-_lib_impl = torch.library.Library("lvar", "IMPL", "CUDA")
-_lib_impl.impl("dense_attn", _dense_attn)
-_lib_impl.impl("dense_colsum_attn", _dense_colsum_attn)
-_lib_impl.impl("csp_attn", _csp_attn)
+_IMPLS = {"dense_attn": _dense_attn, "dense_colsum_attn": _dense_colsum_attn, "csp_attn": _csp_attn}
+
+
+def register_as(namespace: str) -> None:
+    """Registers the three ops under ``torch.ops.<namespace>`` (idempotent).  ``register_as("chipmunk")`` makes
+    the reference's call sites (``torch.ops.chipmunk.dense_attn`` at basic_sparvar.py:384, the ``cuda`` provider
+    branches of sparse_attn_ops.py:55,84,96,289) resolve to this library; it refuses to do so when another
+    extension has already registered one of these ops under that name."""
+    if namespace in _registered:
+        return
+    ns = getattr(torch.ops, namespace)
+    taken = [name for name in _SCHEMAS if hasattr(ns, name)]
+    if taken:
+        raise RuntimeError(f"torch.ops.{namespace} already has {taken}: another extension owns these ops")
+    keep = []
+    native = _lib.torch_binding()
+    frag = torch.library.Library(namespace, "FRAGMENT")
+    for name, schema in _SCHEMAS.items():
+        if name == "dense_attn" and native is not None:
+            native.register_dense_attn(namespace)          # defined and implemented in C++
+            continue
+        frag.define(schema)
+        frag.impl(name, _IMPLS[name], "CUDA")
+    keep.append(frag)
+    _registered[namespace] = keep
+
+
+register_as("lvar")

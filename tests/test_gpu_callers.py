@@ -83,25 +83,92 @@ def test_sparse_diff_attn_full_and_sparse_steps():
 
 
 def test_torch_ops_chipmunk_schemas():
-    import lvar_amd.torch_ops  # noqa: F401
+    """The ops under their default namespace and, after ``register_as("chipmunk")``, under the reference's, called
+    exactly as the reference calls them (basic_sparvar.py:384; sparse_attn_ops.py:55,84,96,289)."""
+    import lvar_amd.torch_ops as tops
+    tops.register_as("chipmunk")
+    tops.register_as("chipmunk")                                            # idempotent
     q, k, v = make_qkv(1, 2, 384, 500, 128, seed=12, amp=0.3)
     qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
-    o, lse = torch.ops.lvar.dense_attn(qg, kg, vg)
     o_ref, M, L = oracle.dense_attn(q, k, v, scale=1.0)
-    assert close(o, o_ref) and lse.shape == (1, 2, 384, 1)
-    # the reference's constant: 1 / (2^M * L)  (dense_attn.cu:227-230)
-    assert torch.allclose(lse.cpu(), 1.0 / (torch.exp2(M) * L), rtol=2e-3)
-    o2, cs, l = torch.ops.lvar.dense_colsum_attn(qg, kg, vg, lse)
     _, cs_ref, _ = oracle.dense_colsum_attn(q, k, v, scale=1.0)
-    assert torch.equal(o2, o) and torch.allclose(cs.cpu(), cs_ref, rtol=2e-3, atol=1e-6) and torch.allclose(l, lse)
     inds = torch.arange(500, dtype=torch.int32).flip(0).expand(1, 2, 2, 500).contiguous()
     counts = torch.full((1, 2, 2), 192, dtype=torch.int32)
-    oc = o.clone()
-    assert torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds.cuda(), counts.cuda(), -1) is None
-    ref = oracle.csp_attn(q, k, v, 1.0, inds, counts, o.cpu(), -1)
-    assert close(oc, ref) and not torch.equal(oc, o)
+    for ns in (torch.ops.lvar, torch.ops.chipmunk):
+        o, lse = ns.dense_attn(qg, kg, vg)
+        assert close(o, o_ref) and lse.shape == (1, 2, 384, 1)
+        # the reference's constant: 1 / (2^M * L)  (dense_attn.cu:227-230)
+        assert torch.allclose(lse.cpu(), 1.0 / (torch.exp2(M) * L), rtol=2e-3)
+        o2, cs, l = ns.dense_colsum_attn(qg, kg, vg, lse)
+        assert torch.equal(o2, o) and torch.allclose(cs.cpu(), cs_ref, rtol=2e-3, atol=1e-6) and torch.allclose(l, lse, rtol=1e-5)
+        oc = o.clone()
+        assert ns.csp_attn(qg, kg, vg, oc, inds.cuda(), counts.cuda(), -1) is None
+        ref = oracle.csp_attn(q, k, v, 1.0, inds, counts, o.cpu(), -1)
+        assert close(oc, ref) and not torch.equal(oc, o)
+        with pytest.raises(Exception):
+            ns.csp_attn(qg, kg, vg, oc, inds.cuda(), counts.cuda(), 2)
+    # the native dense op takes strided inputs (copied) and refuses wrong dtypes
+    qs = qg.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    o3, _ = torch.ops.chipmunk.dense_attn(qs, kg, vg)
+    assert torch.equal(o3, o)
     with pytest.raises(Exception):
-        torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds.cuda(), counts.cuda(), 2)
+        torch.ops.chipmunk.dense_attn(qg.float(), kg, vg)
+    # list checks of the in-place op: int64 lists are refused, lists sliced on the head or group axis are
+    # read through their own strides (copied when they are not the packed ones)
+    oc = o.clone()
+    with pytest.raises(TypeError):
+        torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds.cuda().long(), counts.cuda(), 1)
+    with pytest.raises(TypeError):
+        torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds.cuda(), counts.cuda().long(), 1)
+    with pytest.raises(AssertionError):
+        torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds.cuda()[:, :, 0], counts.cuda(), 1)
+    with pytest.raises(AssertionError):
+        torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds.cuda(), counts.cuda()[:, :1], 1)
+    with pytest.raises(AssertionError):
+        torch.ops.lvar.csp_attn(qg, kg, vg, oc, inds, counts.cuda(), 1)                      # list on another device
+    g = torch.Generator().manual_seed(3)
+    wide = torch.randint(0, 500, (1, 4, 3, 500), generator=g, dtype=torch.int32)
+    wcnt = torch.randint(1, 500, (1, 4, 3), generator=g, dtype=torch.int32)
+    sl_i, sl_c = wide[:, 1:3, :2], wcnt[:, 1:3, :2]                                       # head- and group-sliced views
+    assert not sl_i.is_contiguous()
+    oc = o.clone()
+    torch.ops.lvar.csp_attn(qg, kg, vg, oc, wide.cuda()[:, 1:3, :2], wcnt.cuda()[:, 1:3, :2], 1)
+    assert close(oc, oracle.csp_attn(q, k, v, 1.0, sl_i.contiguous(), sl_c.contiguous(), o.cpu(), 1))
+
+
+def test_reference_shaped_callers_construct():
+    """``SparseDiffAttn(layer_num, layer_counter, use_o_cache=True, spsd_scale=...)`` as basic_sparvar.py:255-259
+    constructs it, with the counter advanced once per call; the kernel-level module under the names of
+    kernels/sparse_attn/triton/__init__.py:1-5."""
+    import lvar_amd.sattn_kernels as sattn_triton
+    from lvar_amd import sparse_attn_config as cfg
+    from lvar_amd.sparse_diff_attn import SparseDiffAttn
+
+    class Counter:
+        n = 0
+
+        def increment(self):
+            self.n += 1
+
+    counter = Counter()
+    mod = SparseDiffAttn(3, counter, use_o_cache=True, spsd_scale=10)
+    assert mod.layer_num == 3 and mod.use_o_cache is True and sorted(mod.local_inds) == [11, 12]
+    assert tuple(mod.local_inds[11][0].shape) == (12, 512) and tuple(mod.local_inds[12][0].shape) == (22, 704)   # windows 7, 9; counts in multiples of 64
+    with pytest.raises(TypeError):
+        SparseDiffAttn(3, True)
+    q, k, v = make_qkv(1, 2, 1600, 4121, 128, seed=21, amp=0.5)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    o = mod(qg, kg, vg, None, do_full_step=True, scale_ind=10, layer_ind=3)
+    assert counter.n == 1 and close(o[:, :1], oracle.dense_attn(q[:, :1], k[:, :1], v[:, :1])[0])
+    cfg.reset()
+    # kernel-level names
+    o2, (M, L) = sattn_triton.dense_attn(qg, kg, vg, scale=None)
+    o3, bs, (M3, L3) = sattn_triton.dense_colsum_attn(qg, kg, vg)
+    assert torch.equal(o2, o3) and bs.shape == (1, 2, 9, 4121) and M.shape == (1, 2, 1600, 1)
+    inds, counts = mod.indices, mod.counts
+    delta, (Md, Ld) = sattn_triton.csp_attn(qg, kg, vg, inds, counts, scale=None)
+    d_ref, _, _ = oracle.csp_attn_delta(q[:, :1], k[:, :1], v[:, :1], inds[:, :1].cpu(), counts[:, :1].cpu())
+    assert close(delta[:, :1], d_ref)
 
 
 @pytest.mark.gpu

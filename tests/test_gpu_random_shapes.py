@@ -118,32 +118,56 @@ def test_token_lists_slice_matches_full_launch():
         assert close(big[sl], ref), (b, h)
 
 
-def test_token_lists_fetch_waves_match_six_wave_groups(tmp_path):
-    """A 192-row group runs with six computing waves plus two fetch waves by default and with six waves that do
-    both under LVAR_CSP_WAVES=6 (read once per process, hence the child processes): same arithmetic per row,
-    so the outputs must agree bit for bit."""
-    import os
-    import subprocess
-    import sys
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    code = (
-        "import sys, torch\n"
-        f"sys.path.insert(0, {root!r}); sys.path.insert(0, {os.path.join(root, 'tests')!r})\n"
-        "from conftest import make_qkv\n"
-        "from lvar_amd import sparse_attn_ops as ops\n"
-        "g = torch.Generator().manual_seed(11)\n"
-        "B, H, Lq, Lk, d = 1, 3, 500, 700, 128\n"
-        "q, k, v = make_qkv(B, H, Lq, Lk, d, seed=11, amp=0.5)\n"
-        "G = (Lq + 191) // 192\n"
-        "idx = torch.randint(0, Lk, (B, H, G, Lk), generator=g, dtype=torch.int32)\n"
-        "cnt = torch.randint(0, Lk + 1, (B, H, G), generator=g, dtype=torch.int32)\n"
-        "o0 = (torch.randn(B, H, Lq, d, generator=g) * 0.5).to(torch.bfloat16)\n"
-        "out = ops.csp_attn(q.cuda(), k.cuda(), v.cuda(), None, idx.cuda(), cnt.cuda(), o0.cuda(), -1)\n"
-        "torch.save(out.cpu(), sys.argv[1])\n")
-    outs = []
-    for waves in ("8", "6"):
-        path = str(tmp_path / f"o{waves}.pt")
-        env = dict(os.environ, LVAR_CSP_WAVES=waves)
-        subprocess.run([sys.executable, "-c", code, path], check=True, env=env, timeout=100)
-        outs.append(torch.load(path, weights_only=True))
-    assert torch.equal(outs[0], outs[1])
+def _csp_abi(q, k, v, idx, cnt, o0, group_rows, o_scale):
+    """lvar_csp_attn_fwd through ctypes with an explicit query-group size."""
+    from lvar_amd import _lib
+    from lvar_amd import sparse_attn_ops as ops
+    B, H, Lq, d = q.shape
+    out = torch.empty_like(q)
+    st = _lib.load().lvar_csp_attn_fwd(ops._view(q), ops._view(k), ops._view(v), ops._view(o0), ops._view(out), None, None,
+                                      idx.data_ptr(), cnt.data_ptr(), idx.shape[2], idx.stride(2), group_rows,
+                                      B, H, Lq, k.shape[2], d, float(o_scale), 1.0 / d ** 0.5,
+                                      torch.cuda.current_stream().cuda_stream)
+    return st, out
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_token_lists_every_workgroup_shape(d):
+    """Query groups of 192 rows run as 8-wave workgroups (six computing waves + two fetch waves), other multiples
+    of 96 / 64 rows as 3- / 2-wave workgroups that fetch for themselves.  Each variant against the oracle at its
+    own group size, and, with every 192-row list repeated for its 96- / 64-row parts, bit for bit against each
+    other: the arithmetic of a query row does not depend on the workgroup shape."""
+    from lvar_amd import _lib
+    g = torch.Generator().manual_seed(11 + d)
+    B, H, Lq, Lk = 1, 3, 500, 700
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=11, amp=0.5)
+    o0 = (torch.randn(B, H, Lq, d, generator=g) * 0.5).to(torch.bfloat16)
+    G = (Lq + 191) // 192
+    idx = torch.randint(0, Lk, (B, H, G, Lk), generator=g, dtype=torch.int32)
+    cnt = torch.randint(0, Lk + 1, (B, H, G), generator=g, dtype=torch.int32)
+    cnt[0, 1, 0] = 0
+    qg, kg, vg, og = q.cuda(), k.cuda(), v.cuda(), o0.cuda()
+    outs = {}
+    for rows in (192, 96, 64):
+        rep = 192 // rows
+        idx_r = idx.repeat_interleave(rep, dim=2).contiguous()
+        cnt_r = cnt.repeat_interleave(rep, dim=2).contiguous()
+        st, out = _csp_abi(qg, kg, vg, idx_r.cuda(), cnt_r.cuda(), og, rows, -1)
+        assert st == 0, (rows, st)
+        ref = oracle.csp_attn(q, k, v, None, idx_r, cnt_r, o0, -1, bm=rows)
+        assert close(out, ref), rows
+        outs[rows] = out
+    assert torch.equal(outs[192], outs[96]) and torch.equal(outs[192], outs[64])
+    # independent lists per 64-row group
+    G64 = (Lq + 63) // 64
+    idx64 = torch.randint(0, Lk, (B, H, G64, Lk), generator=g, dtype=torch.int32)
+    cnt64 = torch.randint(0, Lk + 1, (B, H, G64), generator=g, dtype=torch.int32)
+    st, out = _csp_abi(qg, kg, vg, idx64.cuda(), cnt64.cuda(), og, 64, 1)
+    assert st == 0 and close(out, oracle.csp_attn(q, k, v, None, idx64, cnt64, o0, 1, bm=64))
+    # group sizes that no workgroup shape divides are refused, not mis-run
+    lib = _lib.load()
+    for rows in (32, 160, 224):
+        Gr = (Lq + rows - 1) // rows
+        st, _ = _csp_abi(qg, kg, vg, torch.zeros(B, H, Gr, Lk, dtype=torch.int32).cuda(),
+                         torch.zeros(B, H, Gr, dtype=torch.int32).cuda(), og, rows, 1)
+        assert st == -2 and b"group" in lib.lvar_status_string(st)
