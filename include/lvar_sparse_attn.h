@@ -5,7 +5,8 @@
  * Every entry point takes raw device pointers, sizes and element strides, launches
  * asynchronously on the HIP stream it is given (a hipStream_t passed as void*, NULL =
  * the default stream) and returns 0 or a negative LVAR_E* code.  No entry point
- * allocates, frees or synchronises.  Tensors are bf16 with unit stride on the head
+ * allocates, frees or synchronises; scratch memory, where an entry point uses any, is a
+ * workspace argument.  Tensors are bf16 with unit stride on the head
  * dimension; "strides" are in elements for (batch, head, row).
  *
  * Base-2 softmax statistics follow the reference kernels: M = max_n(q.k*scale*log2e),
@@ -33,6 +34,38 @@ typedef struct {
   int64_t stride_row;
 } lvar_tensor_t;
 
+/*
+ * Partial-result workspace of the balanced launches (the *_ws_fwd entry points): device memory owned by the
+ * caller, 256-byte aligned, that must be all zero before its first use (the library leaves its counters zero
+ * after every launch).  With it, a launch whose plain grid would fill the chip unevenly (fewer than four
+ * rounds of workgroups, e.g. the middle scales of a next-scale-prediction schedule, ragged block lists) runs as
+ * one workgroup per resident slot of the chip instead, each walking an equal share of all tile lists; a query
+ * tile cut between workgroups is finished by the one that arrives last, which adds the pieces up in launch
+ * order, so results are deterministic (they differ from the plain launch in the last bits of fp32 partial
+ * sums only).  A null ptr, or a workspace too small for one slot pair per compute unit, gives the plain launch.
+ * Launches that share a workspace must not overlap in time (one workspace per stream).
+ * min_share_tiles / min_piece_tiles (0 = defaults 8 / 4, in 64-key tiles): the work a workgroup should at
+ * least get, and the smallest piece a query tile may be cut into.
+ * The reference has no counterpart: its kernels launch one program per 64-row query tile
+ * (kernels/sparse_attn/triton/attn_dense.py:205-206, attn_csp.py:236-237).
+ */
+typedef struct {
+  void* ptr;
+  int64_t bytes;
+  int min_share_tiles;
+  int min_piece_tiles;
+} lvar_workspace_t;
+
+/* Bytes of a workspace that lets every balanced launch of the current device use all its slots
+ * (head_dim 64 or 128), or a negative LVAR_E* code. */
+int64_t lvar_attn_workspace_bytes(int head_dim);
+
+/* Workgroups a *_ws_fwd launch of these sizes would run as a balanced launch on the current device, 0 if it
+ * would run as the plain launch; kind 0 = dense, 1 = block list (block_k 64 or 128, list_len = nk_max),
+ * 2 = token list (group_rows, list_len = idx_row_stride).  Pure planning: nothing is launched. */
+int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, int H, int Lq, int Lk, int list_len,
+                                  int head_dim, lvar_workspace_t workspace);
+
 /* Library version (major*10000 + minor*100 + patch) and the gfx target it was built for. */
 int lvar_version(void);
 const char* lvar_target_arch(void);
@@ -51,6 +84,13 @@ int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_
                         float* M, float* L, float* LSE2,
                         int B, int H, int Lq, int Lk, int head_dim,
                         float scale, void* stream);
+
+/* lvar_dense_attn_fwd with a partial-result workspace (see lvar_workspace_t); o must not be NULL for the
+ * workspace to be used. */
+int lvar_dense_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o,
+                           float* M, float* L, float* LSE2,
+                           int B, int H, int Lq, int Lk, int head_dim,
+                           float scale, lvar_workspace_t workspace, void* stream);
 
 /*
  * Dense flash-attention forward returning the per-row constant of the reference's native op:
@@ -102,6 +142,14 @@ int lvar_csp_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v,
                       int B, int H, int Lq, int Lk, int head_dim,
                       float o_scale, float scale, void* stream);
 
+/* lvar_csp_attn_fwd with a partial-result workspace (see lvar_workspace_t). */
+int lvar_csp_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v,
+                         lvar_tensor_t o_accum, lvar_tensor_t o, float* M, float* L,
+                         const int32_t* indices, const int32_t* counts,
+                         int G, int64_t idx_row_stride, int group_rows,
+                         int B, int H, int Lq, int Lk, int head_dim,
+                         float o_scale, float scale, lvar_workspace_t workspace, void* stream);
+
 /*
  * Token-list attention of a sparse step with the O-cache resampled in the epilogue:
  *   o[b,h,i,:] = bilinear(o_cache[b,h])(y_i, x_i) + o_scale * softmax(q_i k[idx]^T scale) v[idx],
@@ -122,6 +170,15 @@ int lvar_csp_attn_upsample_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
                                int B, int H, int Lq, int Lk, int head_dim,
                                float o_scale, float scale, void* stream);
 
+/* lvar_csp_attn_upsample_fwd with a partial-result workspace (see lvar_workspace_t). */
+int lvar_csp_attn_upsample_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v,
+                                  lvar_tensor_t o_cache, int src_side, int dst_side,
+                                  lvar_tensor_t o, float* M, float* L,
+                                  const int32_t* indices, const int32_t* counts,
+                                  int G, int64_t idx_row_stride, int group_rows,
+                                  int B, int H, int Lq, int Lk, int head_dim,
+                                  float o_scale, float scale, lvar_workspace_t workspace, void* stream);
+
 /*
  * Block-sparse attention over a compacted per-query-block list of key blocks in the flex
  * BlockMask layout consumed by SparseFlexAttn (models/sparvar/basic_sparvar.py:55-72,187-194):
@@ -139,6 +196,16 @@ int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
                                int block_q, int block_k,
                                int B, int H, int Lq, int Lk, int head_dim,
                                float scale, void* stream);
+
+/* lvar_block_sparse_attn_fwd with a partial-result workspace (see lvar_workspace_t). */
+int lvar_block_sparse_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o,
+                                  float* M, float* L,
+                                  const int32_t* kv_num_blocks, int64_t stride_nb_b, int64_t stride_nb_h,
+                                  const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
+                                  int64_t stride_ki_q, int nk_max,
+                                  int block_q, int block_k,
+                                  int B, int H, int Lq, int Lk, int head_dim,
+                                  float scale, lvar_workspace_t workspace, void* stream);
 
 /*
  * Block-list build: for every (batch, head, query block) row of block_scores (fp32 contiguous

@@ -14,6 +14,8 @@ EXPORTED_SYMBOLS = (
     "lvar_version", "lvar_target_arch", "lvar_status_string",
     "lvar_dense_attn_fwd", "lvar_dense_attn_rcp_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_csp_attn_upsample_fwd",
     "lvar_block_sparse_attn_fwd",
+    "lvar_attn_workspace_bytes", "lvar_attn_balanced_workgroups", "lvar_dense_attn_ws_fwd", "lvar_csp_attn_ws_fwd", "lvar_csp_attn_upsample_ws_fwd",
+    "lvar_block_sparse_attn_ws_fwd",
     "lvar_block_topk_lists", "lvar_topk_token_lists", "lvar_remap_concat_lists", "lvar_mask_to_lists",
     "lvar_window_key_scores",
 )
@@ -21,6 +23,10 @@ EXPORTED_SYMBOLS = (
 
 class LvarTensor(C.Structure):
     _fields_ = [("ptr", C.c_void_p), ("stride_b", C.c_int64), ("stride_h", C.c_int64), ("stride_row", C.c_int64)]
+
+
+class LvarWorkspace(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("bytes", C.c_int64), ("min_share_tiles", C.c_int), ("min_piece_tiles", C.c_int)]
 
 
 class LvarError(RuntimeError):
@@ -61,6 +67,19 @@ def load() -> C.CDLL:
     lib.lvar_csp_attn_upsample_fwd.argtypes = [T, T, T, T, I, I, T, P, P, P, P, I, I64, I, I, I, I, I, I, F, F, P]
     lib.lvar_block_sparse_attn_fwd.restype = I
     lib.lvar_block_sparse_attn_fwd.argtypes = [T, T, T, T, P, P, P, I64, I64, P, I64, I64, I64, I, I, I, I, I, I, I, I, F, P]
+    W = LvarWorkspace
+    lib.lvar_attn_workspace_bytes.restype = I64
+    lib.lvar_attn_workspace_bytes.argtypes = [I]
+    lib.lvar_attn_balanced_workgroups.restype = I
+    lib.lvar_attn_balanced_workgroups.argtypes = [I, I, I, I, I, I, I, I, I, W]
+    lib.lvar_dense_attn_ws_fwd.restype = I
+    lib.lvar_dense_attn_ws_fwd.argtypes = lib.lvar_dense_attn_fwd.argtypes[:-1] + [W, P]
+    lib.lvar_csp_attn_ws_fwd.restype = I
+    lib.lvar_csp_attn_ws_fwd.argtypes = lib.lvar_csp_attn_fwd.argtypes[:-1] + [W, P]
+    lib.lvar_csp_attn_upsample_ws_fwd.restype = I
+    lib.lvar_csp_attn_upsample_ws_fwd.argtypes = lib.lvar_csp_attn_upsample_fwd.argtypes[:-1] + [W, P]
+    lib.lvar_block_sparse_attn_ws_fwd.restype = I
+    lib.lvar_block_sparse_attn_ws_fwd.argtypes = lib.lvar_block_sparse_attn_fwd.argtypes[:-1] + [W, P]
     lib.lvar_block_topk_lists.restype = I
     lib.lvar_block_topk_lists.argtypes = [P, P, P, P, I, I, I, I, I, P]
     lib.lvar_topk_token_lists.restype = I

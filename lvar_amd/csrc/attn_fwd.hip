@@ -25,8 +25,11 @@
 #include <type_traits>
 #include "common.h"
 #include "launch.h"
+#include "sk_partition.h"
 
 namespace lvar {
+
+int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub, int64_t ws_bytes, int& min_share, int& min_piece);
 
 #ifndef LVAR_AHEAD
 #define LVAR_AHEAD 4
@@ -66,11 +69,17 @@ struct Swz {
   __device__ static __forceinline__ int fv(int row) { return (D == 128) ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 };
 
-template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY>
-__global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_kernel(const AttnParams p) {
-  // The body is compiled for the device only: the host pass just needs the launch stub, and it
-  // silently drops the stub when the body uses the LDS-DMA builtins.
+// Context of a balanced launch (see sk_partition.h); unused by the plain launch.
 #if defined(__HIP_DEVICE_COMPILE__)
+struct SkCtx {
+  SkPartition part;
+  int me;   // index of this workgroup among the P taking part
+};
+
+// One query tile w (or, in a balanced launch, the units [u0, u1) of its tile list; `whole` = all of them).
+template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY, bool SK>
+__device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const int w, const int u0, const int u1,
+                                          const bool whole, const SkCtx& sk) {
   // Token lists with 8 waves: waves 0..5 compute (one 192-row group), waves 6 and 7 only fetch -- they read
   // the list, form the gather addresses and issue every K/V fill.  One 6-wave group fills 6 of the 8 wave
   // slots of a CU; the two fetch waves take the idle ones and the compute waves lose ~10 % of their
@@ -87,17 +96,16 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   constexpr int TILE = 64 * ROWB;
   constexpr int OSTR = D * 2 + 16;  // epilogue transpose buffer row stride (bytes)
   static_assert(NCOMP * 32 * OSTR <= 4 * TILE, "epilogue buffer must fit in the K/V buffers");
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
   // LDS map: K buffers at 0 and TILE, V buffers at 2*TILE and 3*TILE
 
-  // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; remap so that each XCD
-  // walks a contiguous range of (batch, head, q-tile) and K/V of one head stay in its L2.
-  const int per_xcd = gridDim.x >> 3;
-  const int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (w >= p.total_wg) return;
   const int bh = w / p.nqt, qt = w - bh * p.nqt;
   const int b = bh / p.H, h = bh - b * p.H;
-  const int tid = threadIdx.x, lane = tid & 63;
+  int tid_ = threadIdx.x;
+  // A balanced launch runs this function in a loop over its items: everything derived from the lane index is
+  // recomputed per item (the empty asm hides that it is loop-invariant), or the compiler keeps the address
+  // arithmetic of the prologue and the epilogue in registers across the key loop and spills there.
+  if (SK) asm volatile("" : "+v"(tid_));
+  const int tid = tid_, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, r = lane & 31;
   const int fwave = NPROD ? wave - NCOMP : wave;   // index among the filling waves (negative: this wave does not fill)
@@ -109,20 +117,28 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   const bool identity = (MODE == MODE_BLOCK) && p.list == nullptr;
   const int32_t* list = nullptr;
   int T, count;
+  int tile0 = 0;   // identity list of a balanced launch: first tile of this piece
   // first four entries of a block list, read together with the count (not after it): one memory
   // round trip less before the first tile can be fetched; entries beyond the count are never used
   int head[4] = {0, 0, 0, 0};
   if (identity) {
     count = (p.Lk + 63) >> 6;
+    if (SK) { tile0 = u0; count = max(0, min(u1, count) - u0); }
     T = count;
   } else {
     list = p.list + b * p.list_sb + h * p.list_sh + (int64_t)g * p.list_sg;
+    const int first = SK ? (MODE == MODE_BLOCK ? u0 : (u0 << 6)) : 0;   // first list entry of this piece
     if (MODE == MODE_BLOCK) {
 #pragma unroll
       for (int i = 0; i < 4; i++)
-        if (i < p.list_len) head[i] = list[i];
+        if (first + i < p.list_len) head[i] = list[first + i];
     }
     count = max(0, min(p.cnt[b * p.cnt_sb + h * p.cnt_sh + g], p.list_len));
+    if (SK) {
+      const int last = (MODE == MODE_BLOCK) ? u1 : (u1 << 6);
+      count = max(0, min(count, last) - first);
+      list += first;
+    }
     T = (MODE == MODE_BLOCK) ? (count << p.sub_shift) : ((count + 63) >> 6);
   }
   const int sub_shift = identity ? 0 : p.sub_shift;
@@ -136,7 +152,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
   float m_ref = NEG_BIG, m_true = -INFINITY, lsum = 0.f;
   const float c = p.c;
 
-  if (T > 0) {
+  if (T > 0) do {
     // raw buffer descriptors of this (batch, head) slice of K and V: base, stride 0, bound = the bytes of
     // the slice (below 2^31, checked on the host), so a fill beyond the last key row reads zeros
     auto make_rsrc = [](const void* base, int bytes) -> i32x4 {
@@ -162,7 +178,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     constexpr int NR = (MODE == MODE_GATHER) ? SLOTS : 1;
     auto prefetch_raw = [&](int t, int (&raw)[NR]) {
       if (MODE == MODE_BLOCK) {
-        raw[0] = identity ? t : list[t >> sub_shift];
+        raw[0] = identity ? t + tile0 : list[t >> sub_shift];
       } else {
 #pragma unroll
         for (int s = 0; s < SLOTS; s++) {
@@ -271,6 +287,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
         for (int s = 0; s < NR; s++) { rows_v[s] = rows_k[s]; rows_k[s] = rows_n[s]; }
       }
       __syncthreads();   // the one after the last tile
+      if (SK) break;     // a balanced launch has more barriers to meet, below and in the next item
       return;
     }
 
@@ -431,7 +448,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       // compiler from regrouping it.  Phase A: QK MFMA j | K-fragment read j+4 | softmax slot j of
       // S(t).  Phase B: PV MFMA j | the two transposing V reads of MFMA j+4 | the last softmax slots
       // of S(t) (first half) or a slice of the row-maximum reduction of S(t+1) (second half).
-      constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = LVAR_AHEAD;
+      constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = SK ? 2 : LVAR_AHEAD;
       const char* kbuf = smem + (1 - PAR) * TILE;
       const char* vbuf = smem + (2 + PAR) * TILE;
       auto kread = [&](int j) -> bf16x8 {
@@ -564,6 +581,78 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
     } else {
       last(P0{}, sa0, sa1);
     }
+  } while (false);
+
+  if constexpr (SK) {
+    if (!whole) {
+      // ---- a piece of a query tile: park the unnormalised state in this workgroup's workspace slot; the
+      // workgroup whose piece completes the tile adds all pieces up, in launch order, and runs the epilogue ----
+      constexpr int SLOT_FLOATS = D * 32 * NCOMP + 3 * 64 * NCOMP;
+      const bool computes = !(NPROD && wave >= NCOMP);
+      if (computes) {
+        float* slot = p.sk_slots + (int64_t)sk_slot(sk.me, u0 == 0) * SLOT_FLOATS;
+#pragma unroll
+        for (int m = 0; m < MTD; m++)
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            f32x4 v4 = {oacc[m][4 * a], oacc[m][4 * a + 1], oacc[m][4 * a + 2], oacc[m][4 * a + 3]};
+            *(f32x4*)(slot + ((m * 4 + a) * NCOMP + wave) * 256 + lane * 4) = v4;
+          }
+        float* st = slot + D * 32 * NCOMP + wave * 64 + lane;
+        st[0] = m_ref;
+        st[64 * NCOMP] = lsum;
+        st[128 * NCOMP] = m_true;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      __syncthreads();
+      const int lo = sk.part.pfx[w], hi = sk.part.pfx[w + 1];
+      volatile int* flag = (volatile int*)smem;   // the K/V buffers are idle from here on
+      if (tid == 0) {
+        const int n = u1 - u0;
+        const int old = __hip_atomic_fetch_add(p.sk_counters + w, n, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        flag[0] = (old + n == hi - lo) ? 1 : 0;
+      }
+      __syncthreads();
+      const bool finisher = flag[0] != 0;
+      __syncthreads();   // everyone has read the flag before the epilogue reuses the buffer
+      if (!finisher) return;
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      if (tid == 0) __hip_atomic_store(p.sk_counters + w, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+      if (computes) {
+        int j_first, n_inside;
+        sk.part.cuts_inside(w, j_first, n_inside);
+        // pass 1: common reference maximum; pass 2: sum in launch order
+        float m_star = NEG_BIG;
+        m_true = -INFINITY;
+        for (int kp = 0; kp <= n_inside; kp++) {
+          const float* st = p.sk_slots + (int64_t)sk_slot(j_first - 1 + kp, kp == 0) * SLOT_FLOATS + D * 32 * NCOMP + wave * 64 + lane;
+          m_star = fmaxf(m_star, st[0]);
+          m_true = fmaxf(m_true, st[128 * NCOMP]);
+        }
+#pragma unroll
+        for (int m = 0; m < MTD; m++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) oacc[m][i] = 0.f;
+        lsum = 0.f;
+        for (int kp = 0; kp <= n_inside; kp++) {
+          const float* slot = p.sk_slots + (int64_t)sk_slot(j_first - 1 + kp, kp == 0) * SLOT_FLOATS;
+          const float* st = slot + D * 32 * NCOMP + wave * 64 + lane;
+          const float alpha = fast_exp2(st[0] - m_star);
+          lsum += st[64 * NCOMP] * alpha;
+#pragma unroll
+          for (int m = 0; m < MTD; m++)
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+              const f32x4 v4 = *(const f32x4*)(slot + ((m * 4 + a) * NCOMP + wave) * 256 + lane * 4);
+              oacc[m][4 * a] += v4[0] * alpha;
+              oacc[m][4 * a + 1] += v4[1] * alpha;
+              oacc[m][4 * a + 2] += v4[2] * alpha;
+              oacc[m][4 * a + 3] += v4[3] * alpha;
+            }
+        }
+        m_ref = m_star;
+      }
+    }
   }
 
   // ---- epilogue ----
@@ -647,7 +736,110 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
       *(u32x4*)(op + (int64_t)grow * p.o_sr + ocol * 8) = val;
     }
   }
+}
 #endif  // __HIP_DEVICE_COMPILE__
+
+template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY>
+__global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_kernel(const AttnParams p) {
+  // The body is compiled for the device only: the host pass just needs the launch stub, and it
+  // silently drops the stub when the body uses the LDS-DMA builtins.
+#if defined(__HIP_DEVICE_COMPILE__)
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; remap so that each XCD
+  // walks a contiguous range of (batch, head, q-tile) and K/V of one head stay in its L2.
+  const int per_xcd = gridDim.x >> 3;
+  const int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (w >= p.total_wg) return;
+  attn_item<D, NWAVES, MODE, ACCUM, LSE_ONLY, false>(p, smem, w, 0, 0, true, SkCtx{});
+#endif
+}
+
+// Balanced launch: P workgroups (one per resident slot of the chip) split the tile lists of all query tiles
+// into P nearly equal ranges; see sk_partition.h.
+template <int D, int NWAVES, int MODE, bool ACCUM>
+__global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_balanced_kernel(const AttnParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int NPROD = (MODE == MODE_GATHER && NWAVES == 8) ? 2 : 0;
+  constexpr int WGROWS = (NWAVES - NPROD) * 32;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  __shared__ int pfx[SK_MAX_QTILES + 1];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int N = p.total_wg;
+  // weight of every query tile: the entries of its list, at least 1
+  for (int u = tid; u < N; u += NWAVES * 64) {
+    int units;
+    if (MODE == MODE_BLOCK && p.list == nullptr) {
+      units = (p.Lk + 63) >> 6;
+    } else {
+      const int bh = u / p.nqt, qt = u - bh * p.nqt;
+      const int b = bh / p.H, h = bh - b * p.H;
+      const int g = (qt * WGROWS) / p.group_rows;
+      const int cnt = max(0, min(p.cnt[b * p.cnt_sb + h * p.cnt_sh + g], p.list_len));
+      units = (MODE == MODE_BLOCK) ? cnt : ((cnt + 63) >> 6);
+    }
+    pfx[u + 1] = max(units, 1);
+  }
+  __syncthreads();
+  if (wave == 0) {
+    // inclusive scan in place: every lane owns a run of consecutive tiles
+    const int per = (N + 63) >> 6;
+    const int first = lane * per;
+    int sum = 0;
+    for (int j = 0; j < per; j++)
+      if (first + j < N) sum += pfx[first + j + 1];
+    int incl = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    int run = incl - sum;
+    for (int j = 0; j < per; j++)
+      if (first + j < N) {
+        run += pfx[first + j + 1];
+        pfx[first + j + 1] = run;
+      }
+    if (lane == 0) pfx[0] = 0;
+  }
+  __syncthreads();
+  SkCtx sk;
+  sk.part.pfx = pfx;
+  sk.part.N = N;
+  sk.part.U = __builtin_amdgcn_readfirstlane(pfx[N]);
+  sk.part.min_piece = p.sk_min_piece;
+  // no more workgroups than shares of sk_min_share units; if that leaves fewer than one and a half per query tile,
+  // cutting cannot shorten the longest walk: one workgroup per query tile, all tiles whole
+  int P = max(1, min((int)gridDim.x, sk.part.U / p.sk_min_share));
+  if (N <= (int)gridDim.x && 2 * P < 3 * N) {
+    const int me = blockIdx.x;
+    if (me >= N) return;
+    sk.part.P = N;
+    sk.me = me;
+    attn_item<D, NWAVES, MODE, ACCUM, false, true>(p, smem, me, 0, __builtin_amdgcn_readfirstlane(pfx[me + 1] - pfx[me]), true, sk);
+    return;
+  }
+  sk.part.P = P;
+  // With every workgroup taking part, consecutive ranges go to the same XCD (the K/V of a head stay in its L2
+  // and the pieces of a query tile meet there); with fewer, plain order spreads them over all XCDs.
+  const int per_xcd = gridDim.x >> 3;
+  sk.me = (P == (int)gridDim.x) ? (int)((blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3)) : (int)blockIdx.x;
+  if (sk.me >= P) return;
+  int x0 = __builtin_amdgcn_readfirstlane(sk.part.bound(sk.me));
+  const int x1 = __builtin_amdgcn_readfirstlane(sk.part.bound(sk.me + 1));
+  if (x0 >= x1) return;
+  int wq = __builtin_amdgcn_readfirstlane(sk.part.find(x0));
+  bool first_item = true;
+  while (x0 < x1) {
+    const int lo = __builtin_amdgcn_readfirstlane(pfx[wq]), hi = __builtin_amdgcn_readfirstlane(pfx[wq + 1]);
+    const int e = min(x1, hi);
+    if (!first_item) __syncthreads();   // the previous item's epilogue is done with the LDS buffers
+    attn_item<D, NWAVES, MODE, ACCUM, false, true>(p, smem, wq, x0 - lo, e - lo, x0 == lo && e == hi, sk);
+    first_item = false;
+    x0 = e;
+    wq++;
+  }
+#endif
 }
 
 template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY>
@@ -659,6 +851,26 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
   if (p.group_rows % WGROWS != 0) return LVAR_EINVAL;
   p.nqt = (p.Lq + WGROWS - 1) / WGROWS;
   p.total_wg = p.B * p.H * p.nqt;
+  if constexpr (!LSE_ONLY) {
+    // Balanced launch when the caller brought a workspace and the plain grid would leave the chip unevenly
+    // filled: fewer than four rounds of workgroups.  One workgroup per resident slot (two per CU for the 4-wave
+    // kernels), or one per CU if the workspace only holds that many slots.
+    const int64_t per_tile = (MODE == MODE_BLOCK) ? (p.list ? p.list_len : (p.Lk + 63) / 64) : (p.list_len + 63) / 64;
+    const int sub = (MODE == MODE_BLOCK && p.list) ? p.sub_shift : 0;
+    p.sk_wgs = p.sk_ws ? sk_plan(p.total_wg, NWAVES, sk_slot_floats(D, MODE, NWAVES), per_tile, sub, p.sk_ws_bytes,
+                                 p.sk_min_share, p.sk_min_piece) : 0;
+    if (p.sk_wgs > 0) {
+      p.sk_counters = (int*)p.sk_ws;
+      p.sk_slots = (float*)((char*)p.sk_ws + SK_COUNTER_BYTES);
+    }
+    if (p.sk_wgs > 0) {
+      auto kern = attn_fwd_balanced_kernel<D, NWAVES, MODE, ACCUM>;
+      static std::atomic<uint64_t> lds_ready_sk{0};
+      if (!ensure_lds_limit((const void*)kern, SMEM, lds_ready_sk)) return LVAR_ELAUNCH;
+      hipLaunchKernelGGL(kern, dim3(p.sk_wgs), dim3(NWAVES * 64), SMEM, stream, p);
+      return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
+    }
+  }
   const int grid = ((p.total_wg + 7) / 8) * 8;
   auto kern = attn_fwd_kernel<D, NWAVES, MODE, ACCUM, LSE_ONLY>;
   static std::atomic<uint64_t> lds_ready{0};
@@ -683,6 +895,47 @@ int launch_attn(const AttnParams& p, int head_dim, int mode, bool accum, bool ls
   if (head_dim == 128) return launch_d<128>(p, mode, accum, lse_only, nwaves, s);
   if (head_dim == 64) return launch_d<64>(p, mode, accum, lse_only, nwaves, s);
   return LVAR_EUNSUPPORTED;
+}
+
+int device_cus() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  const int slot = dev & 63;
+  int n = cached[slot].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+    cached[slot].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+// Workgroups of the balanced launch, or 0 for the plain launch.  Balanced when the plain grid would leave the chip
+// unevenly filled, i.e. fewer than four rounds of workgroups: one workgroup per resident slot (two per CU for the
+// 4-wave kernels), or one per CU if the workspace only holds that many slot pairs.  `per_tile` is an upper bound
+// of the list entries of a query tile; min_share / min_piece come in as 64-key tiles (0 = default) and go out
+// as list entries (a list entry of a 128-key block list is two tiles: sub = 1).
+int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub, int64_t ws_bytes, int& min_share, int& min_piece) {
+  const int cus = device_cus();
+  const int slots = cus * (nwaves <= 4 ? 2 : 1);
+  if (cus < 8 || cus % 8 != 0 || total_wg > SK_MAX_QTILES || total_wg >= 4 * slots || ws_bytes <= SK_COUNTER_BYTES) return 0;
+  const int64_t fit = (ws_bytes - SK_COUNTER_BYTES) / (2 * (int64_t)slot_floats * 4);
+  const int P = fit >= slots ? slots : (fit >= cus ? cus : 0);
+  const int share = min_share > 0 ? min_share : 8, piece = min_piece > 0 ? min_piece : 4;
+  min_piece = (piece >> sub) > 0 ? (piece >> sub) : 1;
+  min_share = (share >> sub) > min_piece ? (share >> sub) : min_piece;   // shares no smaller than pieces
+  // With fewer query tiles than slots the plain launch already runs them all at once, and cutting only pays if
+  // it makes the longest walk shorter: lists of at least one and a half shares (were every list full; the kernel
+  // looks at the real lists and leaves the tiles whole if they are shorter).
+  if (P == 0) return 0;
+  if (total_wg < slots && 2 * per_tile < 3 * (int64_t)min_share) return 0;
+  return P;
+}
+
+// floats of one workspace slot of a balanced launch: the accumulators and three statistics of every lane
+int sk_slot_floats(int head_dim, int mode, int nwaves) {
+  const int ncomp = (mode == MODE_GATHER && nwaves == 8) ? 6 : nwaves;
+  return head_dim * 32 * ncomp + 3 * 64 * ncomp;
 }
 
 }  // namespace lvar

@@ -44,6 +44,16 @@ void fill_qkv(AttnParams& p, const lvar_tensor_t& q, const lvar_tensor_t& k, con
   p.v = (const bf16_t*)v.ptr; p.v_sb = v.stride_b; p.v_sh = v.stride_h; p.v_sr = v.stride_row;
 }
 
+// A workspace makes the launch eligible for the balanced grid; alignment and size are checked here, whether
+// it is used is decided at launch (launch_one in attn_fwd.hip).
+bool attach_workspace(AttnParams& p, const lvar_workspace_t* ws) {
+  if (!ws || !ws->ptr) return true;
+  if ((reinterpret_cast<uintptr_t>(ws->ptr) & 255u) != 0 || ws->bytes < 0 || ws->min_share_tiles < 0 || ws->min_piece_tiles < 0) return false;
+  p.sk_ws = ws->ptr; p.sk_ws_bytes = ws->bytes;
+  p.sk_min_share = ws->min_share_tiles; p.sk_min_piece = ws->min_piece_tiles;
+  return true;
+}
+
 }  // namespace
 
 extern "C" {
@@ -62,7 +72,8 @@ const char* lvar_status_string(int status) {
 }
 
 static int dense_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
-                        float* LSE2, float* RCP, int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
+                        float* LSE2, float* RCP, int B, int H, int Lq, int Lk, int head_dim, float scale,
+                        const lvar_workspace_t* ws, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k)) return LVAR_EINVAL;
   const bool lse_only = (o.ptr == nullptr);
   if (!kv_span_ok(k, Lk, head_dim) || (!lse_only && !kv_span_ok(v, Lk, head_dim))) return LVAR_EINVAL;
@@ -75,18 +86,25 @@ static int dense_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
   p.c = scale * kLog2e; p.o_scale = 1.f;
   p.list = nullptr; p.cnt = nullptr; p.group_rows = 128; p.sub_shift = 0;
+  if (!attach_workspace(p, ws)) return LVAR_EINVAL;
   return launch_attn(p, head_dim, MODE_BLOCK, false, lse_only, 4, (hipStream_t)stream);
 }
 
 int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
                         float* LSE2, int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
-  return dense_common(q, k, v, o, M, L, LSE2, nullptr, B, H, Lq, Lk, head_dim, scale, stream);
+  return dense_common(q, k, v, o, M, L, LSE2, nullptr, B, H, Lq, Lk, head_dim, scale, nullptr, stream);
+}
+
+int lvar_dense_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+                           float* LSE2, int B, int H, int Lq, int Lk, int head_dim, float scale,
+                           lvar_workspace_t workspace, void* stream) {
+  return dense_common(q, k, v, o, M, L, LSE2, nullptr, B, H, Lq, Lk, head_dim, scale, &workspace, stream);
 }
 
 int lvar_dense_attn_rcp_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* rcp,
                             int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
   if (!o.ptr || !rcp) return LVAR_EINVAL;
-  return dense_common(q, k, v, o, nullptr, nullptr, nullptr, rcp, B, H, Lq, Lk, head_dim, scale, stream);
+  return dense_common(q, k, v, o, nullptr, nullptr, nullptr, rcp, B, H, Lq, Lk, head_dim, scale, nullptr, stream);
 }
 
 int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* cs, float* block_sums,
@@ -108,7 +126,7 @@ int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* 
 static int csp_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o_accum, int up_src, int up_dst,
                       lvar_tensor_t o, float* M, float* L, const int32_t* indices, const int32_t* counts, int G,
                       int64_t idx_row_stride, int group_rows, int B, int H, int Lq, int Lk, int head_dim,
-                      float o_scale, float scale, void* stream) {
+                      float o_scale, float scale, const lvar_workspace_t* ws, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
   if (o.stride_row <= 0 || (o_accum.ptr && (!view_ok(o_accum) || o_accum.stride_row <= 0))) return LVAR_EINVAL;
   if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
@@ -131,6 +149,7 @@ static int csp_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_te
   p.up_src = up_src; p.up_dst = up_dst;
   const int nw = gather_waves(group_rows);
   if (nw == 0) return LVAR_EUNSUPPORTED;
+  if (!attach_workspace(p, ws)) return LVAR_EINVAL;
   return launch_attn(p, head_dim, MODE_GATHER, true, false, nw, (hipStream_t)stream);
 }
 
@@ -139,7 +158,20 @@ int lvar_csp_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_te
                       int64_t idx_row_stride, int group_rows, int B, int H, int Lq, int Lk, int head_dim,
                       float o_scale, float scale, void* stream) {
   return csp_common(q, k, v, o_accum, 0, 0, o, M, L, indices, counts, G, idx_row_stride, group_rows, B, H, Lq, Lk,
-                    head_dim, o_scale, scale, stream);
+                    head_dim, o_scale, scale, nullptr, stream);
+}
+
+int lvar_csp_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o_accum, lvar_tensor_t o,
+                         float* M, float* L, const int32_t* indices, const int32_t* counts, int G,
+                         int64_t idx_row_stride, int group_rows, int B, int H, int Lq, int Lk, int head_dim,
+                         float o_scale, float scale, lvar_workspace_t workspace, void* stream) {
+  return csp_common(q, k, v, o_accum, 0, 0, o, M, L, indices, counts, G, idx_row_stride, group_rows, B, H, Lq, Lk,
+                    head_dim, o_scale, scale, &workspace, stream);
+}
+
+static bool upsample_ok(lvar_tensor_t o_cache, int src_side, int dst_side, int Lq) {
+  return o_cache.ptr && src_side > 0 && dst_side > 0 && src_side <= 32768 && dst_side <= 32768 &&
+         (int64_t)dst_side * dst_side == Lq;
 }
 
 int lvar_csp_attn_upsample_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o_cache,
@@ -147,18 +179,26 @@ int lvar_csp_attn_upsample_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
                                const int32_t* indices, const int32_t* counts, int G, int64_t idx_row_stride,
                                int group_rows, int B, int H, int Lq, int Lk, int head_dim,
                                float o_scale, float scale, void* stream) {
-  if (!o_cache.ptr || src_side <= 0 || dst_side <= 0 || src_side > 32768 || dst_side > 32768 ||
-      (int64_t)dst_side * dst_side != Lq)
-    return LVAR_EINVAL;
+  if (!upsample_ok(o_cache, src_side, dst_side, Lq)) return LVAR_EINVAL;
   return csp_common(q, k, v, o_cache, src_side, dst_side, o, M, L, indices, counts, G, idx_row_stride, group_rows,
-                    B, H, Lq, Lk, head_dim, o_scale, scale, stream);
+                    B, H, Lq, Lk, head_dim, o_scale, scale, nullptr, stream);
 }
 
-int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+int lvar_csp_attn_upsample_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o_cache,
+                                  int src_side, int dst_side, lvar_tensor_t o, float* M, float* L,
+                                  const int32_t* indices, const int32_t* counts, int G, int64_t idx_row_stride,
+                                  int group_rows, int B, int H, int Lq, int Lk, int head_dim,
+                                  float o_scale, float scale, lvar_workspace_t workspace, void* stream) {
+  if (!upsample_ok(o_cache, src_side, dst_side, Lq)) return LVAR_EINVAL;
+  return csp_common(q, k, v, o_cache, src_side, dst_side, o, M, L, indices, counts, G, idx_row_stride, group_rows,
+                    B, H, Lq, Lk, head_dim, o_scale, scale, &workspace, stream);
+}
+
+static int block_sparse_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
                                const int32_t* kv_num_blocks, int64_t stride_nb_b, int64_t stride_nb_h,
                                const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
                                int64_t stride_ki_q, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
-                               int head_dim, float scale, void* stream) {
+                               int head_dim, float scale, const lvar_workspace_t* ws, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
   if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
   if (!kv_num_blocks || !kv_indices || nk_max <= 0 || o.stride_row <= 0) return LVAR_EINVAL;
@@ -175,7 +215,59 @@ int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
   p.list_len = nk_max;
   p.group_rows = block_q;
   p.sub_shift = (block_k == 128) ? 1 : 0;
+  if (!attach_workspace(p, ws)) return LVAR_EINVAL;
   return launch_attn(p, head_dim, MODE_BLOCK, false, false, 4, (hipStream_t)stream);
+}
+
+int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+                               const int32_t* kv_num_blocks, int64_t stride_nb_b, int64_t stride_nb_h,
+                               const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
+                               int64_t stride_ki_q, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
+                               int head_dim, float scale, void* stream) {
+  return block_sparse_common(q, k, v, o, M, L, kv_num_blocks, stride_nb_b, stride_nb_h, kv_indices, stride_ki_b, stride_ki_h,
+                             stride_ki_q, nk_max, block_q, block_k, B, H, Lq, Lk, head_dim, scale, nullptr, stream);
+}
+
+int lvar_block_sparse_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+                                  const int32_t* kv_num_blocks, int64_t stride_nb_b, int64_t stride_nb_h,
+                                  const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
+                                  int64_t stride_ki_q, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
+                                  int head_dim, float scale, lvar_workspace_t workspace, void* stream) {
+  return block_sparse_common(q, k, v, o, M, L, kv_num_blocks, stride_nb_b, stride_nb_h, kv_indices, stride_ki_b, stride_ki_h,
+                             stride_ki_q, nk_max, block_q, block_k, B, H, Lq, Lk, head_dim, scale, &workspace, stream);
+}
+
+int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, int H, int Lq, int Lk, int list_len,
+                                  int head_dim, lvar_workspace_t workspace) {
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || (head_dim != 64 && head_dim != 128) || kind < 0 || kind > 2) return LVAR_EINVAL;
+  if (!workspace.ptr) return 0;
+  int nwaves = 4, mode = MODE_BLOCK, sub = 0;
+  int64_t per_tile = (Lk + 63) / 64;
+  if (kind == 1) {
+    if (block_k != 64 && block_k != 128) return LVAR_EUNSUPPORTED;
+    sub = block_k == 128 ? 1 : 0;
+    per_tile = list_len;
+  } else if (kind == 2) {
+    nwaves = gather_waves(group_rows);
+    if (nwaves == 0) return LVAR_EUNSUPPORTED;
+    mode = MODE_GATHER;
+    per_tile = (list_len + 63) / 64;
+  }
+  const int rows = (nwaves == 8 ? 6 : nwaves) * 32;
+  const int64_t tiles = (int64_t)B * H * ((Lq + rows - 1) / rows);
+  if (tiles > 0x7fffffff) return 0;
+  int share = workspace.min_share_tiles, piece = workspace.min_piece_tiles;
+  return sk_plan((int)tiles, nwaves, sk_slot_floats(head_dim, mode, nwaves), per_tile, sub, workspace.bytes, share, piece);
+}
+
+int64_t lvar_attn_workspace_bytes(int head_dim) {
+  if (head_dim != 64 && head_dim != 128) return LVAR_EUNSUPPORTED;
+  const int cus = device_cus();
+  if (cus <= 0) return LVAR_ELAUNCH;
+  // the larger of: two slots per workgroup, two 4-wave workgroups per CU; two slots per 8-wave workgroup, one per CU
+  const int64_t a = 2ll * (2 * cus) * sk_slot_floats(head_dim, MODE_BLOCK, 4) * 4;
+  const int64_t b = 2ll * cus * sk_slot_floats(head_dim, MODE_GATHER, 8) * 4;
+  return SK_COUNTER_BYTES + (a > b ? a : b);
 }
 
 int lvar_block_topk_lists(const float* block_scores, const uint8_t* base_mask, int32_t* kv_num_blocks,

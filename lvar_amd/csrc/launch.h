@@ -35,6 +35,16 @@ struct AttnParams {
   int up_src, up_dst;  // token-list variant: o_accum is an up_src x up_src token grid, bilinearly
                        // resampled to the up_dst x up_dst grid of the queries (0 = o_accum has Lq rows)
   int nqt, total_wg;
+  // balanced launch: workspace handed in by the caller (null = plain launch).  The launch code fills in sk_wgs
+  // (0 = plain launch after all), sk_counters (per-query-tile arrival counters, all zero between launches) and
+  // sk_slots (2 * sk_wgs slots of partial results).
+  void* sk_ws;
+  int64_t sk_ws_bytes;
+  int* sk_counters;
+  float* sk_slots;
+  int sk_wgs;        // workgroups of the balanced launch, a multiple of 8
+  int sk_min_share;  // list entries a workgroup should at least get (fewer workgroups take part otherwise)
+  int sk_min_piece;  // a cut closer than this many list entries to a query-tile boundary is moved onto it
 };
 
 struct ColsumParams {
@@ -111,5 +121,9 @@ int launch_mask_to_lists(const MaskCompactParams& p, hipStream_t s);
 int launch_block_topk_lists(const MaskListParams& p, hipStream_t s);
 int launch_attn(const AttnParams& p, int head_dim, int mode, bool accum, bool lse_only, int nwaves, hipStream_t s);
 int launch_colsum(const ColsumParams& p, int head_dim, hipStream_t s);
+int sk_slot_floats(int head_dim, int mode, int nwaves);
+int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub, int64_t ws_bytes, int& min_share, int& min_piece);
+int device_cus();   // compute units of the current device (cached), 0 on error
+constexpr int64_t SK_COUNTER_BYTES = 8192;   // head of the workspace: one int32 arrival counter per query tile
 
 }  // namespace lvar

@@ -24,7 +24,7 @@ from .sparse_attn_config import get_kernel_config_attn
 
 __all__ = [
     "dense_attn", "dense_colsum_attn", "dense_colsum_attn_s", "dense_colsum_attn_q", "colsum",
-    "csp_attn", "csp_attn_delta", "block_sparse_attn", "block_topk_lists", "ShapeError",
+    "csp_attn", "csp_attn_delta", "block_sparse_attn", "block_topk_lists", "ShapeError", "set_balanced_launch",
 ]
 
 
@@ -109,6 +109,45 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
+# Partial-result workspaces of the balanced launches (``lvar_workspace_t``): one per (device, stream), allocated
+# zero-filled on first use and kept for the life of the process (launches that share one must not overlap).
+_workspaces = {}
+_balanced = True
+_NO_WORKSPACE = _lib.LvarWorkspace(None, 0, 0, 0)
+
+
+def set_balanced_launch(enabled: bool, min_share_tiles: int = 0, min_piece_tiles: int = 0) -> None:
+    """Switches the balanced launches on or off (default on): with them, an attention call whose plain grid would
+    fill the chip unevenly runs as one workgroup per resident slot, each walking an equal share of all tile
+    lists.  ``min_share_tiles`` / ``min_piece_tiles`` override the library defaults (0 = default)."""
+    global _balanced
+    _balanced = bool(enabled)
+    for ws, _ in _workspaces.values():
+        ws.min_share_tiles, ws.min_piece_tiles = int(min_share_tiles), int(min_piece_tiles)
+    _workspaces_defaults[:] = [int(min_share_tiles), int(min_piece_tiles)]
+
+
+_workspaces_defaults = [0, 0]
+
+
+def _workspace(t: torch.Tensor, stream: int):
+    if not _balanced:
+        return _NO_WORKSPACE
+    key = (t.device.index, stream)
+    hit = _workspaces.get(key)
+    if hit is None:
+        if torch.cuda.is_current_stream_capturing():
+            return _NO_WORKSPACE                     # no allocation inside a graph capture: plain launch
+        with _on_device(t):
+            nbytes = int(_lib.load().lvar_attn_workspace_bytes(128))
+            if nbytes <= 0:
+                return _NO_WORKSPACE
+            buf = torch.zeros(nbytes, dtype=torch.uint8, device=t.device)
+        hit = (_lib.LvarWorkspace(buf.data_ptr(), nbytes, _workspaces_defaults[0], _workspaces_defaults[1]), buf)
+        _workspaces[key] = hit
+    return hit[0]
+
+
 def _dense_launch(q, k, v, scale, want_o=True, want_ml=True, want_lse2=False):
     B, H, Lq, d = q.shape
     Lk = k.shape[2]
@@ -118,9 +157,11 @@ def _dense_launch(q, k, v, scale, want_o=True, want_ml=True, want_lse2=False):
         M, L = torch.empty((2, B, H, Lq, 1), dtype=torch.float32, device=q.device).unbind(0)   # one allocation
     lse2 = torch.empty((B, H, Lq), dtype=torch.float32, device=q.device) if want_lse2 else None
     with _on_device(q):
-        st = _lib.load().lvar_dense_attn_fwd(_view(q), _view(k), _view(v if want_o else None), _view(o), _ptr(M), _ptr(L),
-                                            _ptr(lse2), B, H, Lq, Lk, d, _scale(q, scale), _stream(q))
-    _lib.check(st, "lvar_dense_attn_fwd")
+        stream = _stream(q)
+        st = _lib.load().lvar_dense_attn_ws_fwd(_view(q), _view(k), _view(v if want_o else None), _view(o), _ptr(M), _ptr(L),
+                                               _ptr(lse2), B, H, Lq, Lk, d, _scale(q, scale),
+                                               _workspace(q, stream) if want_o else _NO_WORKSPACE, stream)
+    _lib.check(st, "lvar_dense_attn_ws_fwd")
     return o, M, L, lse2
 
 
@@ -240,16 +281,17 @@ def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, u
         M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
         L = torch.empty_like(M)
     with _on_device(q):
+        stream = _stream(q)
         if upsample_from is None:
-            st = _lib.load().lvar_csp_attn_fwd(_view(q), _view(k), _view(v), _view(o_accum), _view(o), _ptr(M), _ptr(L),
-                                              indices.data_ptr(), counts.data_ptr(), G, indices.stride(2), bm,
-                                              B, H, Lq, Lk, d, float(o_scale), _scale(q, scale), _stream(q))
+            st = _lib.load().lvar_csp_attn_ws_fwd(_view(q), _view(k), _view(v), _view(o_accum), _view(o), _ptr(M), _ptr(L),
+                                                 indices.data_ptr(), counts.data_ptr(), G, indices.stride(2), bm,
+                                                 B, H, Lq, Lk, d, float(o_scale), _scale(q, scale), _workspace(q, stream), stream)
         else:
-            st = _lib.load().lvar_csp_attn_upsample_fwd(
+            st = _lib.load().lvar_csp_attn_upsample_ws_fwd(
                 _view(q), _view(k), _view(v), _view(o_accum), int(upsample_from[0]), int(upsample_from[1]), _view(o),
                 _ptr(M), _ptr(L), indices.data_ptr(), counts.data_ptr(), G, indices.stride(2), bm,
-                B, H, Lq, Lk, d, float(o_scale), _scale(q, scale), _stream(q))
-    _lib.check(st, "lvar_csp_attn_fwd" if upsample_from is None else "lvar_csp_attn_upsample_fwd")
+                B, H, Lq, Lk, d, float(o_scale), _scale(q, scale), _workspace(q, stream), stream)
+    _lib.check(st, "lvar_csp_attn_ws_fwd" if upsample_from is None else "lvar_csp_attn_upsample_ws_fwd")
     return o, M, L
 
 
@@ -315,11 +357,12 @@ def block_sparse_attn(q, k, v, kv_num_blocks, kv_indices, block_q: int = 128, bl
     M = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
     L = torch.empty_like(M)
     with _on_device(q):
-        st = _lib.load().lvar_block_sparse_attn_fwd(
+        stream = _stream(q)
+        st = _lib.load().lvar_block_sparse_attn_ws_fwd(
             _view(q), _view(k), _view(v), _view(o), M.data_ptr(), L.data_ptr(),
             kv_num_blocks.data_ptr(), nb_sb, nb_sh, kv_indices.data_ptr(), ki_sb, ki_sh, kv_indices.stride(2), kv_indices.shape[3],
-            block_q, block_k, B, H, Lq, Lk, d, _scale(q, scale), _stream(q))
-    _lib.check(st, "lvar_block_sparse_attn_fwd")
+            block_q, block_k, B, H, Lq, Lk, d, _scale(q, scale), _workspace(q, stream), stream)
+    _lib.check(st, "lvar_block_sparse_attn_ws_fwd")
     return o, (M, L)
 
 
