@@ -72,8 +72,9 @@ struct Swz {
 // Context of a balanced launch (see sk_partition.h); unused by the plain launch.
 #if defined(__HIP_DEVICE_COMPILE__)
 struct SkCtx {
-  SkPartition part;
-  int me;   // index of this workgroup among the P taking part
+  int j_first, n_inside;   // kept cuts inside this item's query tile
+  int kp;                  // which piece of the tile this item is (0 .. n_inside)
+  int tile_units;          // weight of the whole tile
 };
 
 // One query tile w (or, in a balanced launch, the units [u0, u1) of its tile list; `whole` = all of them).
@@ -100,12 +101,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
 
   const int bh = w / p.nqt, qt = w - bh * p.nqt;
   const int b = bh / p.H, h = bh - b * p.H;
-  int tid_ = threadIdx.x;
-  // A balanced launch runs this function in a loop over its items: everything derived from the lane index is
-  // recomputed per item (the empty asm hides that it is loop-invariant), or the compiler keeps the address
-  // arithmetic of the prologue and the epilogue in registers across the key loop and spills there.
-  if (SK) asm volatile("" : "+v"(tid_));
-  const int tid = tid_, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, r = lane & 31;
   const int fwave = NPROD ? wave - NCOMP : wave;   // index among the filling waves (negative: this wave does not fill)
@@ -287,7 +283,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
         for (int s = 0; s < NR; s++) { rows_v[s] = rows_k[s]; rows_k[s] = rows_n[s]; }
       }
       __syncthreads();   // the one after the last tile
-      if (SK) break;     // a balanced launch has more barriers to meet, below and in the next item
+      if (SK) break;     // a balanced launch has more barriers to meet below
       return;
     }
 
@@ -448,7 +444,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       // compiler from regrouping it.  Phase A: QK MFMA j | K-fragment read j+4 | softmax slot j of
       // S(t).  Phase B: PV MFMA j | the two transposing V reads of MFMA j+4 | the last softmax slots
       // of S(t) (first half) or a slice of the row-maximum reduction of S(t+1) (second half).
-      constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = SK ? 2 : LVAR_AHEAD;
+      constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = LVAR_AHEAD;
       const char* kbuf = smem + (1 - PAR) * TILE;
       const char* vbuf = smem + (2 + PAR) * TILE;
       auto kread = [&](int j) -> bf16x8 {
@@ -585,12 +581,12 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
 
   if constexpr (SK) {
     if (!whole) {
-      // ---- a piece of a query tile: park the unnormalised state in this workgroup's workspace slot; the
-      // workgroup whose piece completes the tile adds all pieces up, in launch order, and runs the epilogue ----
+      // ---- a piece of a query tile: park the unnormalised state in the piece's workspace slot; the workgroup
+      // whose piece completes the tile adds all pieces up, in list order, and runs the epilogue ----
       constexpr int SLOT_FLOATS = D * 32 * NCOMP + 3 * 64 * NCOMP;
       const bool computes = !(NPROD && wave >= NCOMP);
       if (computes) {
-        float* slot = p.sk_slots + (int64_t)sk_slot(sk.me, u0 == 0) * SLOT_FLOATS;
+        float* slot = p.sk_slots + (int64_t)sk_slot(sk.j_first, sk.kp) * SLOT_FLOATS;
 #pragma unroll
         for (int m = 0; m < MTD; m++)
 #pragma unroll
@@ -605,12 +601,11 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
       __syncthreads();
-      const int lo = sk.part.pfx[w], hi = sk.part.pfx[w + 1];
       volatile int* flag = (volatile int*)smem;   // the K/V buffers are idle from here on
       if (tid == 0) {
         const int n = u1 - u0;
         const int old = __hip_atomic_fetch_add(p.sk_counters + w, n, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        flag[0] = (old + n == hi - lo) ? 1 : 0;
+        flag[0] = (old + n == sk.tile_units) ? 1 : 0;
       }
       __syncthreads();
       const bool finisher = flag[0] != 0;
@@ -619,13 +614,11 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
       if (tid == 0) __hip_atomic_store(p.sk_counters + w, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
       if (computes) {
-        int j_first, n_inside;
-        sk.part.cuts_inside(w, j_first, n_inside);
-        // pass 1: common reference maximum; pass 2: sum in launch order
+        // pass 1: common reference maximum; pass 2: sum in list order
         float m_star = NEG_BIG;
         m_true = -INFINITY;
-        for (int kp = 0; kp <= n_inside; kp++) {
-          const float* st = p.sk_slots + (int64_t)sk_slot(j_first - 1 + kp, kp == 0) * SLOT_FLOATS + D * 32 * NCOMP + wave * 64 + lane;
+        for (int kp = 0; kp <= sk.n_inside; kp++) {
+          const float* st = p.sk_slots + (int64_t)sk_slot(sk.j_first, kp) * SLOT_FLOATS + D * 32 * NCOMP + wave * 64 + lane;
           m_star = fmaxf(m_star, st[0]);
           m_true = fmaxf(m_true, st[128 * NCOMP]);
         }
@@ -634,8 +627,8 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
 #pragma unroll
           for (int i = 0; i < 16; i++) oacc[m][i] = 0.f;
         lsum = 0.f;
-        for (int kp = 0; kp <= n_inside; kp++) {
-          const float* slot = p.sk_slots + (int64_t)sk_slot(j_first - 1 + kp, kp == 0) * SLOT_FLOATS;
+        for (int kp = 0; kp <= sk.n_inside; kp++) {
+          const float* slot = p.sk_slots + (int64_t)sk_slot(sk.j_first, kp) * SLOT_FLOATS;
           const float* st = slot + D * 32 * NCOMP + wave * 64 + lane;
           const float alpha = fast_exp2(st[0] - m_star);
           lsum += st[64 * NCOMP] * alpha;
@@ -754,15 +747,18 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
 #endif
 }
 
-// Balanced launch: P workgroups (one per resident slot of the chip) split the tile lists of all query tiles
-// into P nearly equal ranges; see sk_partition.h.
+// Balanced launch: every workgroup runs one item of the partition described in sk_partition.h.  Each workgroup
+// first rebuilds the two prefix tables of the launch in the (still idle) K/V buffers: units before every query
+// tile, and items before every query tile; then it looks up its own item and runs it.
 template <int D, int NWAVES, int MODE, bool ACCUM>
 __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_balanced_kernel(const AttnParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NPROD = (MODE == MODE_GATHER && NWAVES == 8) ? 2 : 0;
   constexpr int WGROWS = (NWAVES - NPROD) * 32;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  __shared__ int pfx[SK_MAX_QTILES + 1];
+  int* pfx = (int*)smem;                  // [N + 1] units before tile u
+  int* ipfx = pfx + SK_MAX_QTILES + 1;    // [N + 1] items before tile u
+  int* found = ipfx + SK_MAX_QTILES + 1;  // the tile of this workgroup's item
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int N = p.total_wg;
@@ -782,7 +778,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_b
   }
   __syncthreads();
   if (wave == 0) {
-    // inclusive scan in place: every lane owns a run of consecutive tiles
+    // both scans by one wave, every lane owning a run of consecutive tiles
     const int per = (N + 63) >> 6;
     const int first = lane * per;
     int sum = 0;
@@ -794,51 +790,60 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_b
       const int up = __shfl_up(incl, d, 64);
       if (lane >= d) incl += up;
     }
-    int run = incl - sum;
+    const int U = __shfl(incl, 63, 64);
+    // share: about one per workgroup slot, none below sk_min_share; with fewer than one and a half shares per query
+    // tile, cutting cannot shorten the longest walk and the tiles stay whole (S = U: no cut anywhere)
+    int S = sk_share(U, p.sk_wgs, p.sk_min_share);
+    if (2 * ((U + S - 1) / S) < 3 * N && N <= p.sk_wgs) S = U;
+    int run = incl - sum, cuts = 0;
     for (int j = 0; j < per; j++)
       if (first + j < N) {
+        const int lo = run;
         run += pfx[first + j + 1];
         pfx[first + j + 1] = run;
+        int jf, ni;
+        sk_cuts_inside(lo, run, S, p.sk_min_piece, jf, ni);
+        ipfx[first + j + 1] = ni;   // for now: cuts inside this tile
+        cuts += ni;
       }
-    if (lane == 0) pfx[0] = 0;
+    int cincl = cuts;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(cincl, d, 64);
+      if (lane >= d) cincl += up;
+    }
+    int crun = cincl - cuts + min(first, N);     // items before this lane's first tile: one per tile plus one per cut
+    for (int j = 0; j < per; j++)
+      if (first + j < N) {
+        crun += ipfx[first + j + 1] + 1;          // items of a tile = cuts inside + 1
+        ipfx[first + j + 1] = crun;
+      }
+    if (lane == 0) { pfx[0] = 0; ipfx[0] = 0; found[1] = S; }
   }
   __syncthreads();
+  const int items = ipfx[N];
+  // consecutive items go to the same XCD (workgroup ids are dealt round-robin to the 8 XCDs): the K/V of a head
+  // stay in its L2 and the pieces of a query tile meet there
+  const int per_xcd = (items + 7) >> 3;
+  const int slot_in_xcd = blockIdx.x >> 3;
+  const int k = (blockIdx.x & 7) * per_xcd + slot_in_xcd;
+  const bool active = slot_in_xcd < per_xcd && k < items;
+  if (active)
+    for (int u = tid; u < N; u += NWAVES * 64)
+      if (ipfx[u] <= k && k < ipfx[u + 1]) found[0] = u;
+  __syncthreads();
+  if (!active) return;
+  const int wq = __builtin_amdgcn_readfirstlane(found[0]);
+  const int S = __builtin_amdgcn_readfirstlane(found[1]);
+  const int lo = __builtin_amdgcn_readfirstlane(pfx[wq]), hi = __builtin_amdgcn_readfirstlane(pfx[wq + 1]);
   SkCtx sk;
-  sk.part.pfx = pfx;
-  sk.part.N = N;
-  sk.part.U = __builtin_amdgcn_readfirstlane(pfx[N]);
-  sk.part.min_piece = p.sk_min_piece;
-  // no more workgroups than shares of sk_min_share units; if that leaves fewer than one and a half per query tile,
-  // cutting cannot shorten the longest walk: one workgroup per query tile, all tiles whole
-  int P = max(1, min((int)gridDim.x, sk.part.U / p.sk_min_share));
-  if (N <= (int)gridDim.x && 2 * P < 3 * N) {
-    const int me = blockIdx.x;
-    if (me >= N) return;
-    sk.part.P = N;
-    sk.me = me;
-    attn_item<D, NWAVES, MODE, ACCUM, false, true>(p, smem, me, 0, __builtin_amdgcn_readfirstlane(pfx[me + 1] - pfx[me]), true, sk);
-    return;
-  }
-  sk.part.P = P;
-  // With every workgroup taking part, consecutive ranges go to the same XCD (the K/V of a head stay in its L2
-  // and the pieces of a query tile meet there); with fewer, plain order spreads them over all XCDs.
-  const int per_xcd = gridDim.x >> 3;
-  sk.me = (P == (int)gridDim.x) ? (int)((blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3)) : (int)blockIdx.x;
-  if (sk.me >= P) return;
-  int x0 = __builtin_amdgcn_readfirstlane(sk.part.bound(sk.me));
-  const int x1 = __builtin_amdgcn_readfirstlane(sk.part.bound(sk.me + 1));
-  if (x0 >= x1) return;
-  int wq = __builtin_amdgcn_readfirstlane(sk.part.find(x0));
-  bool first_item = true;
-  while (x0 < x1) {
-    const int lo = __builtin_amdgcn_readfirstlane(pfx[wq]), hi = __builtin_amdgcn_readfirstlane(pfx[wq + 1]);
-    const int e = min(x1, hi);
-    if (!first_item) __syncthreads();   // the previous item's epilogue is done with the LDS buffers
-    attn_item<D, NWAVES, MODE, ACCUM, false, true>(p, smem, wq, x0 - lo, e - lo, x0 == lo && e == hi, sk);
-    first_item = false;
-    x0 = e;
-    wq++;
-  }
+  sk.kp = k - __builtin_amdgcn_readfirstlane(ipfx[wq]);
+  sk_cuts_inside(lo, hi, S, p.sk_min_piece, sk.j_first, sk.n_inside);
+  sk.tile_units = hi - lo;
+  int u0, u1;
+  sk_piece(lo, hi, S, sk.j_first, sk.n_inside, sk.kp, u0, u1);
+  __syncthreads();   // the tables are dead: the buffers go to the key loop
+  attn_item<D, NWAVES, MODE, ACCUM, false, true>(p, smem, wq, u0, u1, sk.n_inside == 0, sk);
 #endif
 }
 
@@ -867,7 +872,9 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
       auto kern = attn_fwd_balanced_kernel<D, NWAVES, MODE, ACCUM>;
       static std::atomic<uint64_t> lds_ready_sk{0};
       if (!ensure_lds_limit((const void*)kern, SMEM, lds_ready_sk)) return LVAR_ELAUNCH;
-      hipLaunchKernelGGL(kern, dim3(p.sk_wgs), dim3(NWAVES * 64), SMEM, stream, p);
+      // one workgroup per item: at most one per query tile plus one per cut (fewer cuts than shares)
+      const int grid_sk = ((p.total_wg + p.sk_wgs + 7) / 8) * 8;
+      hipLaunchKernelGGL(kern, dim3(grid_sk), dim3(NWAVES * 64), SMEM, stream, p);
       return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
     }
   }
