@@ -36,16 +36,19 @@ typedef struct {
 
 /*
  * Partial-result workspace of the balanced launches (the *_ws_fwd entry points): device memory owned by the
- * caller, 256-byte aligned, that must be all zero before its first use (the library leaves its counters zero
- * after every launch).  With it, a launch whose plain grid would fill the chip unevenly (fewer than four
- * rounds of workgroups, e.g. the middle scales of a next-scale-prediction schedule, ragged block lists) runs as
- * one workgroup per resident slot of the chip instead, each walking an equal share of all tile lists; a query
- * tile cut between workgroups is finished by the one that arrives last, which adds the pieces up in launch
- * order, so results are deterministic (they differ from the plain launch in the last bits of fp32 partial
- * sums only).  A null ptr, or a workspace too small for one slot pair per compute unit, gives the plain launch.
- * Launches that share a workspace must not overlap in time (one workspace per stream).
- * min_share_tiles / min_piece_tiles (0 = defaults 8 / 4, in 64-key tiles): the work a workgroup should at
- * least get, and the smallest piece a query tile may be cut into.
+ * caller, 256-byte aligned, whose first 4096 bytes must be zero before its first use (the library leaves them zero
+ * after every launch).  With it, a launch whose plain grid would fill the chip unevenly (at most 1024 query tiles
+ * and fewer than four rounds of workgroups: the middle scales of a next-scale-prediction schedule, few query tiles
+ * with long or ragged lists) picks a share of about (all list entries) / (resident workgroup slots), cuts every
+ * query tile whose list is long enough into round(entries / share) pieces of equal length and runs one workgroup
+ * per whole tile or piece.  The pieces of a tile are parked in the workspace and added up, in list order, by the
+ * workgroup that arrives last, so results are deterministic (they differ from the plain launch in the last bits
+ * of fp32 partial sums only).  For tile lists the item table of the launch is built on the device from the list
+ * lengths by a one-workgroup kernel ahead of the attention kernel; dense attention needs no table.  A null ptr,
+ * a workspace too small for a slot pair per compute unit, or sizes that leave every query tile whole give the
+ * plain launch.  Launches that share a workspace must not overlap in time (one workspace per stream).
+ * min_share_tiles / min_piece_tiles (0 = defaults 8 / 4, in 64-key tiles): the smallest share, and the
+ * smallest piece a query tile may be cut into.
  * The reference has no counterpart: its kernels launch one program per 64-row query tile
  * (kernels/sparse_attn/triton/attn_dense.py:205-206, attn_csp.py:236-237).
  */

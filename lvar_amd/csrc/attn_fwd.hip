@@ -30,6 +30,7 @@
 namespace lvar {
 
 int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub, int64_t ws_bytes, int& min_share, int& min_piece);
+int64_t sk_plan_bytes(int P);
 
 #ifndef LVAR_AHEAD
 #define LVAR_AHEAD 4
@@ -72,9 +73,10 @@ struct Swz {
 // Context of a balanced launch (see sk_partition.h); unused by the plain launch.
 #if defined(__HIP_DEVICE_COMPILE__)
 struct SkCtx {
-  int j_first, n_inside;   // kept cuts inside this item's query tile
-  int kp;                  // which piece of the tile this item is (0 .. n_inside)
-  int tile_units;          // weight of the whole tile
+  int slot0;        // workspace slot of piece 0 of this item's query tile
+  int pieces;       // pieces of the tile (1 = whole)
+  int kp;           // which piece this item is
+  int tile_units;   // units of the whole tile
 };
 
 // One query tile w (or, in a balanced launch, the units [u0, u1) of its tile list; `whole` = all of them).
@@ -585,62 +587,83 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       // whose piece completes the tile adds all pieces up, in list order, and runs the epilogue ----
       constexpr int SLOT_FLOATS = D * 32 * NCOMP + 3 * 64 * NCOMP;
       const bool computes = !(NPROD && wave >= NCOMP);
+      // The pieces travel between XCDs, whose L2 caches do not see each other's lines.  Rather than writing back
+      // and invalidating whole caches around the exchange (what device-scope fences do), every workspace access is
+      // itself device-coherent: relaxed device-scope atomic stores and loads write through / read past the L2.  The
+      // stores are awaited before the arrival counter is bumped, the loads are issued after its value came back.
+      auto put2 = [](float* dst, float a, float b) {
+        const uint64_t v = (uint64_t)__builtin_bit_cast(uint32_t, a) | ((uint64_t)__builtin_bit_cast(uint32_t, b) << 32);
+        __hip_atomic_store((uint64_t*)dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      };
+      auto get2 = [](const float* src, float& a, float& b) {
+        const uint64_t v = __hip_atomic_load((const uint64_t*)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        a = __builtin_bit_cast(float, (uint32_t)v);
+        b = __builtin_bit_cast(float, (uint32_t)(v >> 32));
+      };
+      auto put1 = [](float* dst, float a) {
+        __hip_atomic_store((uint32_t*)dst, __builtin_bit_cast(uint32_t, a), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      };
+      auto get1 = [](const float* src) -> float {
+        return __builtin_bit_cast(float, __hip_atomic_load((const uint32_t*)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      };
+      // slot layout: accumulator pair (m, i/2) of wave and lane at ((m*8 + i/2)*NCOMP + wave)*128 + lane*2; then
+      // three statistics per lane
       if (computes) {
-        float* slot = p.sk_slots + (int64_t)sk_slot(sk.j_first, sk.kp) * SLOT_FLOATS;
+        float* slot = p.sk_slots + (int64_t)(sk.slot0 + sk.kp) * SLOT_FLOATS;
 #pragma unroll
         for (int m = 0; m < MTD; m++)
 #pragma unroll
-          for (int a = 0; a < 4; a++) {
-            f32x4 v4 = {oacc[m][4 * a], oacc[m][4 * a + 1], oacc[m][4 * a + 2], oacc[m][4 * a + 3]};
-            *(f32x4*)(slot + ((m * 4 + a) * NCOMP + wave) * 256 + lane * 4) = v4;
-          }
+          for (int a = 0; a < 8; a++) put2(slot + ((m * 8 + a) * NCOMP + wave) * 128 + lane * 2, oacc[m][2 * a], oacc[m][2 * a + 1]);
         float* st = slot + D * 32 * NCOMP + wave * 64 + lane;
-        st[0] = m_ref;
-        st[64 * NCOMP] = lsum;
-        st[128 * NCOMP] = m_true;
+        put1(st, m_ref);
+        put1(st + 64 * NCOMP, lsum);
+        put1(st + 128 * NCOMP, m_true);
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // compiler ordering only
+      __builtin_amdgcn_s_waitcnt(0x0f70);                        // vmcnt(0): this wave's stores have been written through
       __syncthreads();
       volatile int* flag = (volatile int*)smem;   // the K/V buffers are idle from here on
       if (tid == 0) {
         const int n = u1 - u0;
-        const int old = __hip_atomic_fetch_add(p.sk_counters + w, n, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int old = __hip_atomic_fetch_add(p.sk_counters + w, n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         flag[0] = (old + n == sk.tile_units) ? 1 : 0;
       }
       __syncthreads();
       const bool finisher = flag[0] != 0;
       __syncthreads();   // everyone has read the flag before the epilogue reuses the buffer
       if (!finisher) return;
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");   // compiler ordering only
       if (tid == 0) __hip_atomic_store(p.sk_counters + w, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
       if (computes) {
-        // pass 1: common reference maximum; pass 2: sum in list order
+        // pass 1: common reference maximum (independent loads, one round trip); pass 2: the pieces in list order,
+        // this workgroup's own included, every one read back from its slot: the same arithmetic whoever finishes
+        const float* st0 = p.sk_slots + (int64_t)sk.slot0 * SLOT_FLOATS + D * 32 * NCOMP + wave * 64 + lane;
         float m_star = NEG_BIG;
         m_true = -INFINITY;
-        for (int kp = 0; kp <= sk.n_inside; kp++) {
-          const float* st = p.sk_slots + (int64_t)sk_slot(sk.j_first, kp) * SLOT_FLOATS + D * 32 * NCOMP + wave * 64 + lane;
-          m_star = fmaxf(m_star, st[0]);
-          m_true = fmaxf(m_true, st[128 * NCOMP]);
-        }
+#pragma unroll
+        for (int kp = 0; kp < SK_MAX_PIECES; kp++)
+          if (kp < sk.pieces) {
+            m_star = fmaxf(m_star, get1(st0 + (int64_t)kp * SLOT_FLOATS));
+            m_true = fmaxf(m_true, get1(st0 + (int64_t)kp * SLOT_FLOATS + 128 * NCOMP));
+          }
 #pragma unroll
         for (int m = 0; m < MTD; m++)
 #pragma unroll
           for (int i = 0; i < 16; i++) oacc[m][i] = 0.f;
         lsum = 0.f;
-        for (int kp = 0; kp <= sk.n_inside; kp++) {
-          const float* slot = p.sk_slots + (int64_t)sk_slot(sk.j_first, kp) * SLOT_FLOATS;
+        for (int kp = 0; kp < sk.pieces; kp++) {
+          const float* slot = p.sk_slots + (int64_t)(sk.slot0 + kp) * SLOT_FLOATS;
           const float* st = slot + D * 32 * NCOMP + wave * 64 + lane;
-          const float alpha = fast_exp2(st[0] - m_star);
-          lsum += st[64 * NCOMP] * alpha;
+          const float alpha = fast_exp2(get1(st) - m_star);
+          lsum = fmaf(get1(st + 64 * NCOMP), alpha, lsum);
 #pragma unroll
           for (int m = 0; m < MTD; m++)
 #pragma unroll
-            for (int a = 0; a < 4; a++) {
-              const f32x4 v4 = *(const f32x4*)(slot + ((m * 4 + a) * NCOMP + wave) * 256 + lane * 4);
-              oacc[m][4 * a] += v4[0] * alpha;
-              oacc[m][4 * a + 1] += v4[1] * alpha;
-              oacc[m][4 * a + 2] += v4[2] * alpha;
-              oacc[m][4 * a + 3] += v4[3] * alpha;
+            for (int a = 0; a < 8; a++) {
+              float x, y;
+              get2(slot + ((m * 8 + a) * NCOMP + wave) * 128 + lane * 2, x, y);
+              oacc[m][2 * a] = fmaf(x, alpha, oacc[m][2 * a]);
+              oacc[m][2 * a + 1] = fmaf(y, alpha, oacc[m][2 * a + 1]);
             }
         }
         m_ref = m_star;
@@ -747,104 +770,126 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_k
 #endif
 }
 
-// Balanced launch: every workgroup runs one item of the partition described in sk_partition.h.  Each workgroup
-// first rebuilds the two prefix tables of the launch in the (still idle) K/V buffers: units before every query
-// tile, and items before every query tile; then it looks up its own item and runs it.
+// Balanced launch: every workgroup runs one item of the partition described in sk_partition.h, which it reads from
+// the item table built by plan_kernel, or, for dense attention (all lists equally long, sk_uniform_n pieces per
+// tile), computes from its index.
 template <int D, int NWAVES, int MODE, bool ACCUM>
 __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_balanced_kernel(const AttnParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int NPROD = (MODE == MODE_GATHER && NWAVES == 8) ? 2 : 0;
-  constexpr int WGROWS = (NWAVES - NPROD) * 32;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  int* pfx = (int*)smem;                  // [N + 1] units before tile u
-  int* ipfx = pfx + SK_MAX_QTILES + 1;    // [N + 1] items before tile u
-  int* found = ipfx + SK_MAX_QTILES + 1;  // the tile of this workgroup's item
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int N = p.total_wg;
-  // weight of every query tile: the entries of its list, at least 1
-  for (int u = tid; u < N; u += NWAVES * 64) {
-    int units;
-    if (MODE == MODE_BLOCK && p.list == nullptr) {
-      units = (p.Lk + 63) >> 6;
-    } else {
-      const int bh = u / p.nqt, qt = u - bh * p.nqt;
-      const int b = bh / p.H, h = bh - b * p.H;
-      const int g = (qt * WGROWS) / p.group_rows;
-      const int cnt = max(0, min(p.cnt[b * p.cnt_sb + h * p.cnt_sh + g], p.list_len));
-      units = (MODE == MODE_BLOCK) ? cnt : ((cnt + 63) >> 6);
-    }
-    pfx[u + 1] = max(units, 1);
-  }
-  __syncthreads();
-  if (wave == 0) {
-    // both scans by one wave, every lane owning a run of consecutive tiles
-    const int per = (N + 63) >> 6;
-    const int first = lane * per;
-    int sum = 0;
-    for (int j = 0; j < per; j++)
-      if (first + j < N) sum += pfx[first + j + 1];
-    int incl = sum;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int up = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += up;
-    }
-    const int U = __shfl(incl, 63, 64);
-    // share: about one per workgroup slot, none below sk_min_share; with fewer than one and a half shares per query
-    // tile, cutting cannot shorten the longest walk and the tiles stay whole (S = U: no cut anywhere)
-    int S = sk_share(U, p.sk_wgs, p.sk_min_share);
-    if (2 * ((U + S - 1) / S) < 3 * N && N <= p.sk_wgs) S = U;
-    int run = incl - sum, cuts = 0;
-    for (int j = 0; j < per; j++)
-      if (first + j < N) {
-        const int lo = run;
-        run += pfx[first + j + 1];
-        pfx[first + j + 1] = run;
-        int jf, ni;
-        sk_cuts_inside(lo, run, S, p.sk_min_piece, jf, ni);
-        ipfx[first + j + 1] = ni;   // for now: cuts inside this tile
-        cuts += ni;
-      }
-    int cincl = cuts;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int up = __shfl_up(cincl, d, 64);
-      if (lane >= d) cincl += up;
-    }
-    int crun = cincl - cuts + min(first, N);     // items before this lane's first tile: one per tile plus one per cut
-    for (int j = 0; j < per; j++)
-      if (first + j < N) {
-        crun += ipfx[first + j + 1] + 1;          // items of a tile = cuts inside + 1
-        ipfx[first + j + 1] = crun;
-      }
-    if (lane == 0) { pfx[0] = 0; ipfx[0] = 0; found[1] = S; }
-  }
-  __syncthreads();
-  const int items = ipfx[N];
+  const bool uniform = p.sk_uniform_n > 0;
+  const int items = uniform ? N * p.sk_uniform_n : min(max(p.sk_plan[1], 0), (int)gridDim.x);
   // consecutive items go to the same XCD (workgroup ids are dealt round-robin to the 8 XCDs): the K/V of a head
   // stay in its L2 and the pieces of a query tile meet there
   const int per_xcd = (items + 7) >> 3;
   const int slot_in_xcd = blockIdx.x >> 3;
   const int k = (blockIdx.x & 7) * per_xcd + slot_in_xcd;
-  const bool active = slot_in_xcd < per_xcd && k < items;
-  if (active)
-    for (int u = tid; u < N; u += NWAVES * 64)
-      if (ipfx[u] <= k && k < ipfx[u + 1]) found[0] = u;
-  __syncthreads();
-  if (!active) return;
-  const int wq = __builtin_amdgcn_readfirstlane(found[0]);
-  const int S = __builtin_amdgcn_readfirstlane(found[1]);
-  const int lo = __builtin_amdgcn_readfirstlane(pfx[wq]), hi = __builtin_amdgcn_readfirstlane(pfx[wq + 1]);
+  if (slot_in_xcd >= per_xcd || k >= items) return;
   SkCtx sk;
-  sk.kp = k - __builtin_amdgcn_readfirstlane(ipfx[wq]);
-  sk_cuts_inside(lo, hi, S, p.sk_min_piece, sk.j_first, sk.n_inside);
-  sk.tile_units = hi - lo;
-  int u0, u1;
-  sk_piece(lo, hi, S, sk.j_first, sk.n_inside, sk.kp, u0, u1);
-  __syncthreads();   // the tables are dead: the buffers go to the key loop
-  attn_item<D, NWAVES, MODE, ACCUM, false, true>(p, smem, wq, u0, u1, sk.n_inside == 0, sk);
+  int w, u0, u1;
+  if (uniform) {
+    const int n = p.sk_uniform_n, T = (p.Lk + 63) >> 6;
+    w = k / n;
+    sk.kp = k - w * n;
+    sk.pieces = n;
+    sk.slot0 = w * n;
+    sk.tile_units = T;
+    sk_piece(T, n, sk.kp, u0, u1);
+  } else {
+    const int* it = p.sk_plan + SK_PLAN_HEADER + SK_PLAN_ITEM * k;
+    w = max(0, min(it[0], N - 1));
+    u0 = it[1];
+    u1 = it[2];
+    sk.slot0 = it[3];
+    sk.pieces = it[4];
+    sk.kp = it[5];
+    sk.tile_units = it[6];
+    // a damaged table must not send a store outside the workspace
+    if (sk.pieces < 1 || sk.pieces > SK_MAX_PIECES || sk.kp < 0 || sk.kp >= sk.pieces || (sk.pieces > 1 && (sk.slot0 < 0 || sk.slot0 + sk.pieces > 2 * p.sk_wgs))) return;
+  }
+  attn_item<D, NWAVES, MODE, ACCUM, false, true>(p, smem, w, u0, u1, sk.pieces == 1, sk);
 #endif
+}
+
+// Item table of a balanced launch over tile lists, from the list lengths: one workgroup.
+template <int WGROWS, int MODE>
+__global__ __launch_bounds__(256) void plan_kernel(const AttnParams p, int* plan) {
+  __shared__ int units[SK_MAX_QTILES];    // units of tile u
+  __shared__ int ipfx[SK_MAX_QTILES + 1]; // items before tile u
+  __shared__ int spfx[SK_MAX_QTILES + 1]; // slots before tile u
+  __shared__ int total[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int N = p.total_wg;
+  for (int u = tid; u < N; u += 256) {
+    const int bh = u / p.nqt, qt = u - bh * p.nqt;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int g = (qt * WGROWS) / p.group_rows;
+    const int cnt = max(0, min(p.cnt[b * p.cnt_sb + h * p.cnt_sh + g], p.list_len));
+    units[u] = (MODE == MODE_BLOCK) ? cnt : ((cnt + 63) >> 6);
+  }
+  __syncthreads();
+  if (wave == 0) {
+    // every lane owns a run of consecutive tiles; U first, then the two prefix tables
+    const int per = (N + 63) >> 6, first = lane * per;
+    int sum = 0;
+    for (int j = 0; j < per; j++)
+      if (first + j < N) sum += max(units[first + j], 1);
+    int U = sum;
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) U += __shfl_xor(U, d, 64);
+    int S = sk_share(U, p.sk_wgs, p.sk_min_share);
+    const bool cut = sk_worth_cutting(U, S, N, p.sk_wgs);
+    int it = 0, sl = 0;
+    for (int j = 0; j < per; j++)
+      if (first + j < N) {
+        const int n = cut ? sk_pieces(units[first + j], S, p.sk_min_piece) : 1;
+        it += n;
+        sl += n > 1 ? n : 0;
+      }
+    int it_incl = it, sl_incl = sl;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int a = __shfl_up(it_incl, d, 64), c = __shfl_up(sl_incl, d, 64);
+      if (lane >= d) { it_incl += a; sl_incl += c; }
+    }
+    int irun = it_incl - it, srun = sl_incl - sl;
+    for (int j = 0; j < per; j++)
+      if (first + j < N) {
+        const int n = cut ? sk_pieces(units[first + j], S, p.sk_min_piece) : 1;
+        ipfx[first + j] = irun;
+        spfx[first + j] = srun;
+        irun += n;
+        srun += n > 1 ? n : 0;
+      }
+    if (lane == 63) { total[0] = it_incl; total[1] = sl_incl; total[2] = S; total[3] = cut ? 1 : 0; }
+  }
+  __syncthreads();
+  const int S = total[2];
+  const bool cut = total[3] != 0;
+  // the pieces-per-share bound keeps both totals inside the launch (N + sk_wgs items) and the workspace (2 * sk_wgs
+  // slots); if a list-length table breaks it after all, every tile stays whole
+  const bool fits = total[0] <= N + p.sk_wgs && total[1] <= 2 * p.sk_wgs;
+  if (tid == 0) {
+    plan[0] = SK_PLAN_MAGIC;
+    plan[1] = fits ? total[0] : N;
+    plan[2] = N;
+    plan[3] = S;
+    plan[4] = fits ? total[1] : 0;
+    plan[5] = plan[6] = plan[7] = 0;
+  }
+  for (int u = tid; u < N; u += 256) {
+    const int T = units[u];
+    const int n = (cut && fits) ? sk_pieces(T, S, p.sk_min_piece) : 1;
+    const int base = fits ? ipfx[u] : u;
+    for (int kp = 0; kp < n; kp++) {
+      int u0, u1;
+      sk_piece(T, n, kp, u0, u1);
+      int* it = plan + SK_PLAN_HEADER + SK_PLAN_ITEM * (base + kp);
+      it[0] = u; it[1] = u0; it[2] = u1; it[3] = n > 1 ? spfx[u] : -1;
+      it[4] = n; it[5] = kp; it[6] = T; it[7] = 0;
+    }
+  }
 }
 
 template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY>
@@ -857,23 +902,38 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
   p.nqt = (p.Lq + WGROWS - 1) / WGROWS;
   p.total_wg = p.B * p.H * p.nqt;
   if constexpr (!LSE_ONLY) {
-    // Balanced launch when the caller brought a workspace and the plain grid would leave the chip unevenly
-    // filled: fewer than four rounds of workgroups.  One workgroup per resident slot (two per CU for the 4-wave
-    // kernels), or one per CU if the workspace only holds that many slots.
+    const bool dense = (MODE == MODE_BLOCK && p.list == nullptr);
     const int64_t per_tile = (MODE == MODE_BLOCK) ? (p.list ? p.list_len : (p.Lk + 63) / 64) : (p.list_len + 63) / 64;
     const int sub = (MODE == MODE_BLOCK && p.list) ? p.sub_shift : 0;
     p.sk_wgs = p.sk_ws ? sk_plan(p.total_wg, NWAVES, sk_slot_floats(D, MODE, NWAVES), per_tile, sub, p.sk_ws_bytes,
                                  p.sk_min_share, p.sk_min_piece) : 0;
-    if (p.sk_wgs > 0) {
-      p.sk_counters = (int*)p.sk_ws;
-      p.sk_slots = (float*)((char*)p.sk_ws + SK_COUNTER_BYTES);
+    p.sk_uniform_n = 0;
+    if (p.sk_wgs > 0 && dense) {
+      // all lists have (Lk + 63) / 64 entries: the pieces per tile follow from the sizes alone
+      const int T = (int)per_tile, U = p.total_wg * T;
+      const int S = sk_share(U, p.sk_wgs, p.sk_min_share);
+      const int n = sk_worth_cutting(U, S, p.total_wg, p.sk_wgs) ? sk_pieces(T, S, p.sk_min_piece) : 1;
+      if (n > 1 && (int64_t)n * p.total_wg <= 2 * p.sk_wgs) p.sk_uniform_n = n; else p.sk_wgs = 0;   // whole tiles: the plain launch
     }
     if (p.sk_wgs > 0) {
+      p.sk_counters = (int*)p.sk_ws;
+      p.sk_slots = (float*)((char*)p.sk_ws + SK_COUNTER_BYTES + sk_plan_bytes(p.sk_wgs));
+      int grid_sk;
+      if (p.sk_uniform_n > 0) {
+        grid_sk = ((p.total_wg * p.sk_uniform_n + 7) / 8) * 8;
+      } else {
+        if (!p.sk_plan) {
+          // no table from the caller: build it now, in the workspace
+          int* plan = (int*)((char*)p.sk_ws + SK_COUNTER_BYTES);
+          hipLaunchKernelGGL((plan_kernel<WGROWS, MODE>), dim3(1), dim3(256), 0, stream, p, plan);
+          if (hipGetLastError() != hipSuccess) return LVAR_ELAUNCH;
+          p.sk_plan = plan;
+        }
+        grid_sk = ((p.total_wg + p.sk_wgs + 7) / 8) * 8;   // at most one item per query tile plus one per share
+      }
       auto kern = attn_fwd_balanced_kernel<D, NWAVES, MODE, ACCUM>;
       static std::atomic<uint64_t> lds_ready_sk{0};
       if (!ensure_lds_limit((const void*)kern, SMEM, lds_ready_sk)) return LVAR_ELAUNCH;
-      // one workgroup per item: at most one per query tile plus one per cut (fewer cuts than shares)
-      const int grid_sk = ((p.total_wg + p.sk_wgs + 7) / 8) * 8;
       hipLaunchKernelGGL(kern, dim3(grid_sk), dim3(NWAVES * 64), SMEM, stream, p);
       return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
     }
@@ -926,8 +986,9 @@ int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub
   const int cus = device_cus();
   const int slots = cus * (nwaves <= 4 ? 2 : 1);
   if (cus < 8 || cus % 8 != 0 || total_wg > SK_MAX_QTILES || total_wg >= 4 * slots || ws_bytes <= SK_COUNTER_BYTES) return 0;
-  const int64_t fit = (ws_bytes - SK_COUNTER_BYTES) / (2 * (int64_t)slot_floats * 4);
-  const int P = fit >= slots ? slots : (fit >= cus ? cus : 0);
+  if (per_tile * total_wg >= (1ll << 30)) return 0;   // unit counts stay well inside 32 bits
+  auto fits = [&](int P) { return SK_COUNTER_BYTES + sk_plan_bytes(P) + 2 * (int64_t)P * slot_floats * 4 <= ws_bytes; };
+  const int P = fits(slots) ? slots : (fits(cus) ? cus : 0);
   const int share = min_share > 0 ? min_share : 8, piece = min_piece > 0 ? min_piece : 4;
   min_piece = (piece >> sub) > 0 ? (piece >> sub) : 1;
   min_share = (share >> sub) > min_piece ? (share >> sub) : min_piece;   // shares no smaller than pieces
@@ -937,6 +998,12 @@ int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub
   if (P == 0) return 0;
   if (total_wg < slots && 2 * per_tile < 3 * (int64_t)min_share) return 0;
   return P;
+}
+
+// bytes of the item-table area of a workspace for P shares (256-byte granules)
+int64_t sk_plan_bytes(int P) {
+  const int64_t b = (int64_t)(SK_PLAN_HEADER + SK_PLAN_ITEM * (SK_MAX_QTILES + P)) * 4;
+  return (b + 255) / 256 * 256;
 }
 
 // floats of one workspace slot of a balanced launch: the accumulators and three statistics of every lane

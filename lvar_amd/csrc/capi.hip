@@ -264,9 +264,9 @@ int64_t lvar_attn_workspace_bytes(int head_dim) {
   if (head_dim != 64 && head_dim != 128) return LVAR_EUNSUPPORTED;
   const int cus = device_cus();
   if (cus <= 0) return LVAR_ELAUNCH;
-  // the larger of: two slots per workgroup, two 4-wave workgroups per CU; two slots per 8-wave workgroup, one per CU
-  const int64_t a = 2ll * (2 * cus) * sk_slot_floats(head_dim, MODE_BLOCK, 4) * 4;
-  const int64_t b = 2ll * cus * sk_slot_floats(head_dim, MODE_GATHER, 8) * 4;
+  // the larger of: two slots per share with two 4-wave workgroups per CU, or with one 8-wave workgroup per CU
+  const int64_t a = sk_plan_bytes(2 * cus) + 2ll * (2 * cus) * sk_slot_floats(head_dim, MODE_BLOCK, 4) * 4;
+  const int64_t b = sk_plan_bytes(cus) + 2ll * cus * sk_slot_floats(head_dim, MODE_GATHER, 8) * 4;
   return SK_COUNTER_BYTES + (a > b ? a : b);
 }
 

@@ -42,7 +42,9 @@ struct AttnParams {
   int64_t sk_ws_bytes;
   int* sk_counters;
   float* sk_slots;
-  int sk_wgs;        // workgroups of the balanced launch, a multiple of 8
+  int sk_wgs;        // shares of the balanced launch (resident workgroup slots it is planned for)
+  const int* sk_plan;  // item table (plan_kernel), from the caller or built in the workspace; unused for dense attention
+  int sk_uniform_n;  // dense attention: pieces per query tile (0 = use the table)
   int sk_min_share;  // list entries a workgroup should at least get (fewer workgroups take part otherwise)
   int sk_min_piece;  // a cut closer than this many list entries to a query-tile boundary is moved onto it
 };
@@ -124,6 +126,7 @@ int launch_colsum(const ColsumParams& p, int head_dim, hipStream_t s);
 int sk_slot_floats(int head_dim, int mode, int nwaves);
 int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub, int64_t ws_bytes, int& min_share, int& min_piece);
 int device_cus();   // compute units of the current device (cached), 0 on error
-constexpr int64_t SK_COUNTER_BYTES = 8192;   // head of the workspace: one int32 arrival counter per query tile
+constexpr int64_t SK_COUNTER_BYTES = 4096;   // head of the workspace: one int32 arrival counter per query tile
+int64_t sk_plan_bytes(int P);                // then the item table, then 2 * P slots
 
 }  // namespace lvar
