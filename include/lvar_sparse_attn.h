@@ -25,6 +25,7 @@ extern "C" {
 #define LVAR_EINVAL (-1)      /* bad size / null pointer / misaligned pointer or stride */
 #define LVAR_EUNSUPPORTED (-2) /* head_dim, block shape or query-group size not built */
 #define LVAR_ELAUNCH (-3)      /* HIP reported a launch error */
+#define LVAR_ETOOBIG (-4)      /* lvar_block_sparse_attn_static_fwd: more query tiles than its scratch buffer holds */
 
 /* Tensor view: base pointer plus element strides of a [B,H,rows,d] bf16 tensor (d stride 1). */
 typedef struct {
@@ -209,6 +210,28 @@ int lvar_block_sparse_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_
                                   int block_q, int block_k,
                                   int B, int H, int Lq, int Lk, int head_dim,
                                   float scale, lvar_workspace_t workspace, void* stream);
+
+/*
+ * lvar_block_sparse_attn_ws_fwd without the workspace argument: the partial-result workspace is a buffer of
+ * LVAR_STATIC_SCRATCH_BYTES that lives inside the library (one copy per GPU, held until the process ends), so this
+ * entry point allocates nothing and takes no memory beyond the inputs and outputs from the caller.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments, results and balanced-launch
+ * rule as lvar_block_sparse_attn_ws_fwd given a zeroed workspace of LVAR_STATIC_SCRATCH_BYTES.
+ * Limits: B * H * ceil(Lq / 128) <= LVAR_STATIC_MAX_QUERY_TILES and head_dim <= 128, else LVAR_ETOOBIG (larger
+ * launches have enough query tiles to fill the chip: use lvar_block_sparse_attn_fwd).  All calls on one GPU share
+ * that GPU's buffer: calls that overlap in time on one GPU (different streams or threads) race.
+ */
+#define LVAR_STATIC_SCRATCH_BYTES (34ll << 20)
+#define LVAR_STATIC_MAX_QUERY_TILES 1024
+int lvar_block_sparse_attn_static_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o,
+                                      float* M, float* L,
+                                      const int32_t* kv_num_blocks, int64_t stride_nb_b, int64_t stride_nb_h,
+                                      const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
+                                      int64_t stride_ki_q, int nk_max,
+                                      int block_q, int block_k,
+                                      int B, int H, int Lq, int Lk, int head_dim,
+                                      float scale, void* stream);
 
 /*
  * Block-list build: for every (batch, head, query block) row of block_scores (fp32 contiguous

@@ -15,7 +15,7 @@ EXPORTED_SYMBOLS = (
     "lvar_dense_attn_fwd", "lvar_dense_attn_rcp_fwd", "lvar_colsum_fwd", "lvar_csp_attn_fwd", "lvar_csp_attn_upsample_fwd",
     "lvar_block_sparse_attn_fwd",
     "lvar_attn_workspace_bytes", "lvar_attn_balanced_workgroups", "lvar_dense_attn_ws_fwd", "lvar_csp_attn_ws_fwd", "lvar_csp_attn_upsample_ws_fwd",
-    "lvar_block_sparse_attn_ws_fwd",
+    "lvar_block_sparse_attn_ws_fwd", "lvar_block_sparse_attn_static_fwd",
     "lvar_block_topk_lists", "lvar_topk_token_lists", "lvar_remap_concat_lists", "lvar_mask_to_lists",
     "lvar_window_key_scores",
 )
@@ -80,6 +80,8 @@ def load() -> C.CDLL:
     lib.lvar_csp_attn_upsample_ws_fwd.argtypes = lib.lvar_csp_attn_upsample_fwd.argtypes[:-1] + [W, P]
     lib.lvar_block_sparse_attn_ws_fwd.restype = I
     lib.lvar_block_sparse_attn_ws_fwd.argtypes = lib.lvar_block_sparse_attn_fwd.argtypes[:-1] + [W, P]
+    lib.lvar_block_sparse_attn_static_fwd.restype = I
+    lib.lvar_block_sparse_attn_static_fwd.argtypes = lib.lvar_block_sparse_attn_fwd.argtypes
     lib.lvar_block_topk_lists.restype = I
     lib.lvar_block_topk_lists.argtypes = [P, P, P, P, I, I, I, I, I, P]
     lib.lvar_topk_token_lists.restype = I

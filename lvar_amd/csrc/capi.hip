@@ -6,7 +6,32 @@
 
 using namespace lvar;
 
+// Scratch of lvar_block_sparse_attn_static_fwd: arrival counters, item table and partial-result slots of a balanced
+// launch with one share per compute unit of a 256-CU part at head_dim 128 (4 KiB + 41 KiB + 2 * 256 * 67 KiB).
+// Every GPU the library runs on holds its own copy, at its own address, until the process ends.  In host code the
+// name is only a handle for hipGetSymbolAddress: the address that kernels and fills take is looked up per device.
+constexpr int64_t kStaticScratchBytes = 34ll << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
+
+// words [0, n) of a device buffer := 0 (a kernel, not hipMemsetAsync: callers may be capturing a HIP graph)
+__global__ void zero_words_kernel(uint32_t* dst, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = 0u;
+}
+
+// Device address of this GPU's copy of `scratch`, looked up once per device with that device current.
+void* static_scratch() {
+  static std::atomic<void*> ptrs[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  void* ptr = ptrs[dev].load(std::memory_order_acquire);
+  if (ptr) return ptr;
+  if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return nullptr;
+  ptrs[dev].store(ptr, std::memory_order_release);
+  return ptr;
+}
 
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -67,6 +92,7 @@ const char* lvar_status_string(int status) {
     case LVAR_EINVAL: return "invalid argument (size, null/misaligned pointer, stride or scale)";
     case LVAR_EUNSUPPORTED: return "unsupported head_dim, block shape or query-group size";
     case LVAR_ELAUNCH: return "HIP launch failed";
+    case LVAR_ETOOBIG: return "problem larger than the static scratch buffer allows (use the workspace entry point)";
     default: return "unknown status";
   }
 }
@@ -258,6 +284,29 @@ int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, 
   if (tiles > 0x7fffffff) return 0;
   int share = workspace.min_share_tiles, piece = workspace.min_piece_tiles;
   return sk_plan((int)tiles, nwaves, sk_slot_floats(head_dim, mode, nwaves), per_tile, sub, workspace.bytes, share, piece);
+}
+
+int lvar_block_sparse_attn_static_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+                                      const int32_t* kv_num_blocks, int64_t stride_nb_b, int64_t stride_nb_h,
+                                      const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
+                                      int64_t stride_ki_q, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
+                                      int head_dim, float scale, void* stream) {
+  if (B <= 0 || H <= 0 || Lq <= 0) return LVAR_EINVAL;
+  // the scratch holds the counters and the item table of at most LVAR_STATIC_MAX_QUERY_TILES query tiles
+  const int64_t tiles = (int64_t)B * H * ((Lq + 127) / 128);
+  if (tiles > LVAR_STATIC_MAX_QUERY_TILES || head_dim > 128) return LVAR_ETOOBIG;
+  void* ptr = static_scratch();
+  if (!ptr) return LVAR_ELAUNCH;
+  // The array keeps what the last call left: the arrival counters must start at zero (they do after a launch that
+  // ran to its end; a fill makes that independent of the past).
+  hipLaunchKernelGGL(zero_words_kernel, dim3((int)(SK_COUNTER_BYTES / 4 / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (uint32_t*)ptr, (int)(SK_COUNTER_BYTES / 4));
+  if (hipGetLastError() != hipSuccess) return LVAR_ELAUNCH;
+  lvar_workspace_t ws{};
+  ws.ptr = ptr;
+  ws.bytes = kStaticScratchBytes;
+  return block_sparse_common(q, k, v, o, M, L, kv_num_blocks, stride_nb_b, stride_nb_h, kv_indices, stride_ki_b, stride_ki_h,
+                             stride_ki_q, nk_max, block_q, block_k, B, H, Lq, Lk, head_dim, scale, &ws, stream);
 }
 
 int64_t lvar_attn_workspace_bytes(int head_dim) {
