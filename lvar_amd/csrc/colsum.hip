@@ -32,8 +32,14 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
   const int per_xcd = gridDim.x >> 3;
   const int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (w >= p.total_wg) return;
-  const int bh = w / p.nkt, kt = w - bh * p.nkt;
+  // workgroup = (batch*head, key tile of 256 keys, range of query groups): the query axis is cut at group
+  // boundaries when the plain grid would fill the chip unevenly; every range writes its own groups of cs
+  const int per_bh = p.nkt * p.q_splits;
+  const int bh = w / per_bh, rem = w - bh * per_bh;
+  const int kt = rem / p.q_splits, sp = rem - kt * p.q_splits;
   const int b = bh / p.H, h = bh - b * p.H;
+  const int qoff = __builtin_amdgcn_readfirstlane(sp * p.split_rows);   // first query row of this range (a multiple of 64 and of group_rows)
+  const int Lq_l = min(p.Lq, qoff + p.split_rows) - qoff;   // rows of this range
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hh = lane >> 5, r = lane & 31;
@@ -73,12 +79,12 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
   const int fill_voff = fill_trow0 * q_srb + ((lcs ^ ((fill_trow0 / (256 / ROWB)) & (CPR - 1))) << 4);
   auto issue_stage = [&](int s) {
     const uint32_t dst = lds0 + (s & (NSTAGE - 1)) * QTILE;
-    if (s * 64 + 64 <= p.Lq) {
+    if (s * 64 + 64 <= Lq_l) {
       // all 64 rows exist: constant lane offset, stage and slot move the scalar offset
 #pragma unroll
       for (int sl = 0; sl < SLOTS; sl++) {
         const int i = wave + sl * 4;
-        const int soff = (s * 64 + sl * 4 * RPI) * q_srb;
+        const int soff = (qoff + s * 64 + sl * 4 * RPI) * q_srb;
         const uint32_t m0v = dst + i * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(m0v), "v"(fill_voff), "s"(qrsrc), "s"(soff) : "memory");
       }
@@ -87,14 +93,14 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
       for (int sl = 0; sl < SLOTS; sl++) {
         const int i = wave + sl * 4;
         const int trow = i * RPI + lrow;
-        const int grow = min(s * 64 + trow, p.Lq - 1);
+        const int grow = min(qoff + s * 64 + trow, p.Lq - 1);
         const int voff = grow * q_srb + ((lcs ^ ((trow / (256 / ROWB)) & (CPR - 1))) << 4);
         const uint32_t m0v = dst + i * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(m0v), "v"(voff), "s"(qrsrc) : "memory");
       }
     }
     if (wave == 0) {
-      const int voff = min(s * 64 + lane, p.Lq - 1) * 4;
+      const int voff = min(qoff + s * 64 + lane, p.Lq - 1) * 4;
       const uint32_t m0v = lds0 + LSE_OFF + (s & (NLSE - 1)) * 256;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(m0v), "v"(voff), "s"(lrsrc) : "memory");
     }
@@ -131,8 +137,8 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
     }
   };
 
-  const int S = (p.Lq + 63) >> 6;          // stages
-  const int U = (p.Lq + 31) >> 5;          // 32-row tiles
+  const int S = (Lq_l + 63) >> 6;          // stages of this range
+  const int U = (Lq_l + 31) >> 5;          // 32-row tiles
   const int kbase_l = r * ROWB + ((hh ^ ((r / (256 / ROWB)) & (CPR - 1))) << 4);
   float acc[2] = {0.f, 0.f};
 
@@ -142,8 +148,8 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
     f32x4 lse[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) lse[j] = *(const f32x4*)(ll + j * 32);
-    const bool ragged = (u * 32 + 32 > p.Lq);
-    const int lim = p.Lq - u * 32 - 4 * hh;
+    const bool ragged = (u * 32 + 32 > Lq_l);
+    const int lim = Lq_l - u * 32 - 4 * hh;
     float pa = 0.f, pb = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
@@ -160,7 +166,7 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
     acc[0] += pa;
     acc[1] += pb;
     const int qend = u * 32 + 32;
-    if (qend % p.group_rows == 0 || qend >= p.Lq) flush((u * 32) / p.group_rows, acc);
+    if (qend % p.group_rows == 0 || qend >= Lq_l) flush((qoff + u * 32) / p.group_rows, acc);
   };
 
   // prologue: up to three stages in flight
@@ -230,7 +236,7 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
       acc[0] += pa;
       acc[1] += pb;
       const int qend = up * 32 + 32;
-      if (qend % p.group_rows == 0) flush((up * 32) / p.group_rows, acc);
+      if (qend % p.group_rows == 0) flush((qoff + up * 32) / p.group_rows, acc);
     } else {
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
@@ -262,7 +268,25 @@ static int launch_cs(const ColsumParams& p0, hipStream_t stream) {
   ColsumParams p = p0;
   p.nkb = (p.Lk + 63) / 64;
   p.nkt = (p.Lk + 255) / 256;
-  p.total_wg = p.B * p.H * p.nkt;
+  // Ranges of query groups per key tile.  With fewer than four rounds of workgroups on the chip's resident slots
+  // (two per CU) the last, partly filled round costs as much as a full one: cut the query axis so that the rounds
+  // get shorter.  Cost model: rounds x (64-row stages per range + 3 stages' worth of fixed cost per workgroup).
+  const int unit = (p.group_rows % 64 == 0) ? p.group_rows : (p.group_rows % 32 == 0 ? 2 * p.group_rows : 0);   // lcm(group_rows, 64)
+  p.q_splits = 1;
+  p.split_rows = ((p.Lq + 63) / 64) * 64 + (unit > 0 ? unit : 64);   // one range covers everything
+  const int base_wg = p.B * p.H * p.nkt, slots = 2 * device_cus();
+  if (unit > 0 && slots > 0 && base_wg < 4 * slots) {
+    const int units_total = (p.Lq + unit - 1) / unit;
+    int64_t best = -1;
+    for (int s = 1; s <= 8 && s <= units_total; s++) {
+      const int rows = ((units_total + s - 1) / s) * unit;          // rows per range
+      const int n = (p.Lq + rows - 1) / rows;                       // ranges that hold rows
+      const int64_t rounds = ((int64_t)base_wg * n + slots - 1) / slots;
+      const int64_t cost = rounds * ((rows + 63) / 64 + 3);
+      if (best < 0 || cost < best) { best = cost; p.q_splits = n; p.split_rows = rows; }
+    }
+  }
+  p.total_wg = base_wg * p.q_splits;
   const int grid = ((p.total_wg + 7) / 8) * 8;
   constexpr int SMEM = 4 * 64 * D * 2 + 8 * 256;
   static std::atomic<uint64_t> lds_ready{0};

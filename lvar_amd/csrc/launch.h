@@ -60,6 +60,7 @@ struct ColsumParams {
   int group_rows;
   float c;
   int nkt, nkb, total_wg;
+  int q_splits, split_rows;   // ranges of query groups per key tile, rows per range (set at launch)
 };
 
 struct MaskListParams {
