@@ -82,18 +82,20 @@ const char* lvar_status_string(int status);
  * (kernels/sparse_attn/triton/attn_dense.py:186-231).
  * LSE2, if not NULL, receives the base-2 log-sum-exp M + log2(L) (fp32 [B,H,Lq]), the form the
  * colsum entry point consumes.  o may be NULL (statistics only); M, L and LSE2 may each be NULL.
- * head_dim in {64, 128}.
+ * head_dim in {64, 128}.  Grouped-query attention: k and v hold kv_heads heads, H a multiple of it, and query
+ * head h reads K/V head h / (H / kv_heads) (the layout of the reference's expansion, kernels/sparse_attn/
+ * sparse_attn_ops.py:228-233; kernels/chipmunk/csrc/attn/dense_colsum_attn.cu:386-387); kv_heads = H otherwise.
  */
 int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o,
                         float* M, float* L, float* LSE2,
-                        int B, int H, int Lq, int Lk, int head_dim,
+                        int B, int H, int kv_heads, int Lq, int Lk, int head_dim,
                         float scale, void* stream);
 
 /* lvar_dense_attn_fwd with a partial-result workspace (see lvar_workspace_t); o must not be NULL for the
  * workspace to be used. */
 int lvar_dense_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o,
                            float* M, float* L, float* LSE2,
-                           int B, int H, int Lq, int Lk, int head_dim,
+                           int B, int H, int kv_heads, int Lq, int Lk, int head_dim,
                            float scale, lvar_workspace_t workspace, void* stream);
 
 /*
@@ -103,7 +105,7 @@ int lvar_dense_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lv
  * torch.ops.chipmunk.dense_colsum_attn takes as its fourth argument.  o and rcp must not be NULL.
  */
 int lvar_dense_attn_rcp_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* rcp,
-                            int B, int H, int Lq, int Lk, int head_dim,
+                            int B, int H, int kv_heads, int Lq, int Lk, int head_dim,
                             float scale, void* stream);
 
 /*
@@ -116,10 +118,11 @@ int lvar_dense_attn_rcp_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, l
  * Replaces pass 2 of _full_attn_fwd (kernels/sparse_attn/triton/attn_dense_colsum.py:216-231)
  * and torch.ops.chipmunk.dense_colsum_attn (kernels/chipmunk/csrc/chipmunk.cu:58,
  * kernels/chipmunk/csrc/attn/dense_colsum_attn.cu:355-522), which takes the same precomputed
- * per-row constant as its fourth argument.
+ * per-row constant as its fourth argument.  k holds kv_heads heads (grouped-query attention as in
+ * lvar_dense_attn_fwd; the column sums stay per query head).
  */
 int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* cs, float* block_sums,
-                    int B, int H, int Lq, int Lk, int head_dim, int q_group_size,
+                    int B, int H, int kv_heads, int Lq, int Lk, int head_dim, int q_group_size,
                     float scale, void* stream);
 
 /*

@@ -56,11 +56,11 @@ def load() -> C.CDLL:
     lib.lvar_status_string.restype = C.c_char_p
     lib.lvar_status_string.argtypes = [I]
     lib.lvar_dense_attn_fwd.restype = I
-    lib.lvar_dense_attn_fwd.argtypes = [T, T, T, T, P, P, P, I, I, I, I, I, F, P]
+    lib.lvar_dense_attn_fwd.argtypes = [T, T, T, T, P, P, P, I, I, I, I, I, I, F, P]
     lib.lvar_dense_attn_rcp_fwd.restype = I
-    lib.lvar_dense_attn_rcp_fwd.argtypes = [T, T, T, T, P, I, I, I, I, I, F, P]
+    lib.lvar_dense_attn_rcp_fwd.argtypes = [T, T, T, T, P, I, I, I, I, I, I, F, P]
     lib.lvar_colsum_fwd.restype = I
-    lib.lvar_colsum_fwd.argtypes = [T, T, P, P, P, I, I, I, I, I, I, F, P]
+    lib.lvar_colsum_fwd.argtypes = [T, T, P, P, P, I, I, I, I, I, I, I, F, P]
     lib.lvar_csp_attn_fwd.restype = I
     lib.lvar_csp_attn_fwd.argtypes = [T, T, T, T, T, P, P, P, P, I, I64, I, I, I, I, I, I, F, F, P]
     lib.lvar_csp_attn_upsample_fwd.restype = I

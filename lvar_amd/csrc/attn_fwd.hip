@@ -161,8 +161,9 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       return rs;
     };
     const int k_srb = (int)p.k_sr * 2, v_srb = (int)p.v_sr * 2;  // row strides in bytes
-    const i32x4 krsrc = make_rsrc(p.k + b * p.k_sb + h * p.k_sh, (p.Lk - 1) * k_srb + ROWB);
-    const i32x4 vrsrc = make_rsrc(p.v + b * p.v_sb + h * p.v_sh, (p.Lk - 1) * v_srb + ROWB);
+    const int hkv = h / p.kv_group;   // grouped-query attention: kv_group query heads share a K/V head
+    const i32x4 krsrc = make_rsrc(p.k + b * p.k_sb + hkv * p.k_sh, (p.Lk - 1) * k_srb + ROWB);
+    const i32x4 vrsrc = make_rsrc(p.v + b * p.v_sb + hkv * p.v_sh, (p.Lk - 1) * v_srb + ROWB);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(LVAR_LDS char*)smem;
 
     // per-lane role in a tile load: row (within the RPI rows of one instruction) and chunk slot
@@ -895,6 +896,7 @@ __global__ __launch_bounds__(256) void plan_kernel(const AttnParams p, int* plan
 template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY>
 static int launch_one(const AttnParams& p0, hipStream_t stream) {
   AttnParams p = p0;
+  if (p.kv_group < 1) p.kv_group = 1;
   constexpr int WGROWS = ((MODE == MODE_GATHER && NWAVES == 8) ? 6 : NWAVES) * 32;   // two of eight token-list waves only fetch
   constexpr int SMEM = 4 * 64 * D * 2;
   if (MODE == MODE_BLOCK && p.list == nullptr) p.group_rows = WGROWS;  // dense: any row grouping

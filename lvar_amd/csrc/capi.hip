@@ -83,7 +83,7 @@ bool attach_workspace(AttnParams& p, const lvar_workspace_t* ws) {
 
 extern "C" {
 
-int lvar_version(void) { return 100; }
+int lvar_version(void) { return 200; }
 const char* lvar_target_arch(void) { return "gfx950"; }
 
 const char* lvar_status_string(int status) {
@@ -98,9 +98,10 @@ const char* lvar_status_string(int status) {
 }
 
 static int dense_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
-                        float* LSE2, float* RCP, int B, int H, int Lq, int Lk, int head_dim, float scale,
+                        float* LSE2, float* RCP, int B, int H, int kv_heads, int Lq, int Lk, int head_dim, float scale,
                         const lvar_workspace_t* ws, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k)) return LVAR_EINVAL;
+  if (kv_heads <= 0 || H % kv_heads != 0) return LVAR_EINVAL;
   const bool lse_only = (o.ptr == nullptr);
   if (!kv_span_ok(k, Lk, head_dim) || (!lse_only && !kv_span_ok(v, Lk, head_dim))) return LVAR_EINVAL;
   if (!lse_only && (!view_ok(v) || !view_ok(o) || o.stride_row <= 0)) return LVAR_EINVAL;
@@ -109,7 +110,7 @@ static int dense_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_
   fill_qkv(p, q, k, lse_only ? k : v);
   p.o = (bf16_t*)o.ptr; p.o_sb = o.stride_b; p.o_sh = o.stride_h; p.o_sr = o.stride_row;
   p.M = M; p.L = L; p.LSE2 = LSE2; p.RCP = RCP;
-  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk; p.kv_group = H / kv_heads;
   p.c = scale * kLog2e; p.o_scale = 1.f;
   p.list = nullptr; p.cnt = nullptr; p.group_rows = 128; p.sub_shift = 0;
   if (!attach_workspace(p, ws)) return LVAR_EINVAL;
@@ -117,32 +118,33 @@ static int dense_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_
 }
 
 int lvar_dense_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
-                        float* LSE2, int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
-  return dense_common(q, k, v, o, M, L, LSE2, nullptr, B, H, Lq, Lk, head_dim, scale, nullptr, stream);
+                        float* LSE2, int B, int H, int kv_heads, int Lq, int Lk, int head_dim, float scale, void* stream) {
+  return dense_common(q, k, v, o, M, L, LSE2, nullptr, B, H, kv_heads, Lq, Lk, head_dim, scale, nullptr, stream);
 }
 
 int lvar_dense_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
-                           float* LSE2, int B, int H, int Lq, int Lk, int head_dim, float scale,
+                           float* LSE2, int B, int H, int kv_heads, int Lq, int Lk, int head_dim, float scale,
                            lvar_workspace_t workspace, void* stream) {
-  return dense_common(q, k, v, o, M, L, LSE2, nullptr, B, H, Lq, Lk, head_dim, scale, &workspace, stream);
+  return dense_common(q, k, v, o, M, L, LSE2, nullptr, B, H, kv_heads, Lq, Lk, head_dim, scale, &workspace, stream);
 }
 
 int lvar_dense_attn_rcp_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* rcp,
-                            int B, int H, int Lq, int Lk, int head_dim, float scale, void* stream) {
+                            int B, int H, int kv_heads, int Lq, int Lk, int head_dim, float scale, void* stream) {
   if (!o.ptr || !rcp) return LVAR_EINVAL;
-  return dense_common(q, k, v, o, nullptr, nullptr, nullptr, rcp, B, H, Lq, Lk, head_dim, scale, nullptr, stream);
+  return dense_common(q, k, v, o, nullptr, nullptr, nullptr, rcp, B, H, kv_heads, Lq, Lk, head_dim, scale, nullptr, stream);
 }
 
 int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* cs, float* block_sums,
-                    int B, int H, int Lq, int Lk, int head_dim, int q_group_size, float scale, void* stream) {
+                    int B, int H, int kv_heads, int Lq, int Lk, int head_dim, int q_group_size, float scale, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !lse2 || !cs) return LVAR_EINVAL;
+  if (kv_heads <= 0 || H % kv_heads != 0) return LVAR_EINVAL;
   if (q_group_size <= 0 || q_group_size % 32 != 0) return LVAR_EINVAL;
   if (!kv_span_ok(q, Lq, head_dim)) return LVAR_EINVAL;
   ColsumParams p{};
   p.q = (const bf16_t*)q.ptr; p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sr = q.stride_row;
   p.k = (const bf16_t*)k.ptr; p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sr = k.stride_row;
   p.lse2 = lse2; p.cs = cs; p.bs = block_sums;
-  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk; p.kv_group = H / kv_heads;
   p.group_rows = q_group_size;
   p.G = (Lq + q_group_size - 1) / q_group_size;
   p.c = scale * kLog2e;

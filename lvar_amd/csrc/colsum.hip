@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
   const float c = p.c;
 
   // stationary K^T fragments: lane holds key column n0 + nt*32 + r, d = ks*16 + 8*hh .. +7
-  const bf16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
+  const bf16_t* kbase = p.k + b * p.k_sb + (h / p.kv_group) * p.k_sh;   // grouped-query attention: shared key heads
   bf16x8 kf[2][KS];
 #pragma unroll
   for (int nt = 0; nt < 2; nt++) {
@@ -266,6 +266,7 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
 template <int D>
 static int launch_cs(const ColsumParams& p0, hipStream_t stream) {
   ColsumParams p = p0;
+  if (p.kv_group < 1) p.kv_group = 1;
   p.nkb = (p.Lk + 63) / 64;
   p.nkt = (p.Lk + 255) / 256;
   // Ranges of query groups per key tile.  With fewer than four rounds of workgroups on the chip's resident slots

@@ -22,6 +22,7 @@ struct AttnParams {
   int64_t o_sb, o_sh, o_sr;
   int64_t oa_sb, oa_sh, oa_sr;
   int B, H, Lq, Lk;
+  int kv_group;   // query heads per key/value head (1 = as many K/V heads as query heads)
   float c;        // softmax scale * log2(e)
   float o_scale;  // epilogue factor of the token-list variant
   // key-tile list: kv_indices / kv_num_blocks (block list) or indices / counts (token list)
@@ -57,6 +58,7 @@ struct ColsumParams {
   int64_t q_sb, q_sh, q_sr;
   int64_t k_sb, k_sh, k_sr;
   int B, H, Lq, Lk, G;
+  int kv_group;   // query heads per key head
   int group_rows;
   float c;
   int nkt, nkb, total_wg;

@@ -51,7 +51,8 @@ void bind(uintptr_t dense_attn_fwd, uintptr_t dense_attn_rcp_fwd) {
 py::object fast_dense_attn(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, std::optional<double> scale) {
   if (!g_dense || !plain(q) || !plain(k) || !plain(v)) return py::none();
   const int64_t B = q.size(0), H = q.size(1), Lq = q.size(2), d = q.size(3), Lk = k.size(2);
-  if (k.sizes() != v.sizes() || k.size(0) != B || k.size(1) != H || k.size(3) != d || (d != 64 && d != 128)) return py::none();
+  const int64_t Hkv = k.size(1);
+  if (k.sizes() != v.sizes() || k.size(0) != B || Hkv <= 0 || H % Hkv != 0 || k.size(3) != d || (d != 64 && d != 128)) return py::none();
   if (Lq <= 0 || Lk <= 0 || B <= 0 || H <= 0 || Lq > INT32_MAX || Lk > INT32_MAX) return py::none();
   const auto dev = q.get_device();
   if (k.get_device() != dev || v.get_device() != dev || c10::hip::current_device() != dev) return py::none();
@@ -61,7 +62,7 @@ py::object fast_dense_attn(const at::Tensor& q, const at::Tensor& k, const at::T
   float* mp = ml.data_ptr<float>();
   void* stream = c10::hip::getCurrentHIPStream(dev).stream();
   const int st = g_dense(view(q), view(k), view(v), view(o), mp, mp + B * H * Lq, nullptr, static_cast<int>(B),
-                         static_cast<int>(H), static_cast<int>(Lq), static_cast<int>(Lk), static_cast<int>(d), s, stream);
+                         static_cast<int>(H), static_cast<int>(Hkv), static_cast<int>(Lq), static_cast<int>(Lk), static_cast<int>(d), s, stream);
   if (st != LVAR_OK) return py::none();   // the general path reports the error
   return py::make_tuple(o, ml.select(0, 0), ml.select(0, 1));
 }
@@ -83,14 +84,15 @@ std::vector<at::Tensor> op_dense_attn(const at::Tensor& q_in, const at::Tensor& 
   const at::Tensor q = as_plain(q_in, "q"), k = as_plain(k_in, "k"), v = as_plain(v_in, "v");
   const int64_t B = q.size(0), H = q.size(1), Lq = q.size(2), d = q.size(3), Lk = k.size(2);
   TORCH_CHECK(k.sizes() == v.sizes(), "k/v shape mismatch: ", k.sizes(), " vs ", v.sizes());
-  TORCH_CHECK(k.size(0) == B && k.size(1) == H && k.size(3) == d, "q/k batch, head or head_dim mismatch: ", q.sizes(), " vs ", k.sizes());
+  const int64_t Hkv = k.size(1);
+  TORCH_CHECK(k.size(0) == B && Hkv > 0 && H % Hkv == 0 && k.size(3) == d, "q/k batch, head or head_dim mismatch: ", q.sizes(), " vs ", k.sizes());
   TORCH_CHECK(q.get_device() == k.get_device() && q.get_device() == v.get_device(), "q, k, v must be on the same device");
   TORCH_CHECK(Lq <= INT32_MAX && Lk <= INT32_MAX, "sequence too long");
   const c10::DeviceGuard guard(q.device());   // the tensors' device is current for the allocations and the launch
   at::Tensor o = at::empty_like(q);
   at::Tensor rcp = at::empty({B, H, Lq, 1}, q.options().dtype(at::kFloat));
   void* stream = c10::hip::getCurrentHIPStream(q.get_device()).stream();
-  const int st = g_dense_rcp(view(q), view(k), view(v), view(o), rcp.data_ptr<float>(), static_cast<int>(B), static_cast<int>(H),
+  const int st = g_dense_rcp(view(q), view(k), view(v), view(o), rcp.data_ptr<float>(), static_cast<int>(B), static_cast<int>(H), static_cast<int>(Hkv),
                              static_cast<int>(Lq), static_cast<int>(Lk), static_cast<int>(d), 1.0f, stream);
   TORCH_CHECK(st == LVAR_OK, "lvar_dense_attn_rcp_fwd failed with status ", st,
               st == LVAR_EUNSUPPORTED ? " (unsupported head_dim)" : st == LVAR_EINVAL ? " (invalid argument)" : " (launch failed)");

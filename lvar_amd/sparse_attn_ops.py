@@ -43,6 +43,23 @@ def _scale(q: torch.Tensor, scale) -> float:
     return 1.0 / math.sqrt(q.shape[-1]) if scale is None else float(scale)
 
 
+def _pad_head_dim(q, k, v=None):
+    """Head dimensions 16 and 32 (the reference's Triton kernels take {16, 32, 64, 128, 256},
+    kernels/sparse_attn/triton/attn_dense_colsum.py:246) run on the 64-wide kernels with zero padding: zero
+    columns add nothing to q.k, and the padded output columns (zero) are cut off again.  Returns the padded
+    tensors and the original head_dim, or the inputs and None when no padding applies."""
+    d = q.shape[-1]
+    if d not in (16, 32) or q.dim() != 4:
+        return q, k, v, None
+    pad = (0, 64 - d)
+    f = torch.nn.functional.pad
+    return f(q, pad), f(k, pad), (None if v is None else f(v, pad)), d
+
+
+def _scale_for(d: int, scale) -> float:
+    return 1.0 / math.sqrt(d) if scale is None else float(scale)
+
+
 def _prep(t: torch.Tensor, name: str) -> torch.Tensor:
     if t.dtype is torch.bfloat16 and t.is_cuda and t.dim() == 4 and t.is_contiguous() and t.shape[-1] % 8 == 0 \
             and t.data_ptr() % 16 == 0:
@@ -63,15 +80,19 @@ def _view(t: Optional[torch.Tensor]) -> _lib.LvarTensor:
     return _lib.LvarTensor(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
 
 
-def _check_qkv(q, k, v):
+def _check_qkv(q, k, v, gqa: bool = False):
+    """``gqa``: the op supports grouped-query attention (fewer K/V heads than query heads, query head ``h`` reads
+    K/V head ``h // (H // Hkv)``: the expansion of the reference's naive_dense_colsum_attn2,
+    kernels/sparse_attn/sparse_attn_ops.py:228-233)."""
     # messages are only formatted on failure: these checks run on every call
     qs, ks = q.shape, k.shape
     if ks != v.shape:
         raise ShapeError(f"k/v shape mismatch: {tuple(k.shape)} vs {tuple(v.shape)}")
-    if qs[0] != ks[0] or qs[1] != ks[1] or qs[3] != ks[3]:
-        raise ShapeError(f"q/k batch, head or head_dim mismatch: {tuple(q.shape)} vs {tuple(k.shape)}")
+    if qs[0] != ks[0] or qs[3] != ks[3] or (qs[1] != ks[1] and not (gqa and ks[1] > 0 and qs[1] % ks[1] == 0)):
+        raise ShapeError(f"q/k batch, head or head_dim mismatch: {tuple(q.shape)} vs {tuple(k.shape)}"
+                         + ("" if gqa or qs[1] == ks[1] else " (this op takes as many K/V heads as query heads)"))
     if qs[3] != 128 and qs[3] != 64:
-        raise ShapeError(f"head_dim must be 64 or 128, got {q.shape[-1]}")
+        raise ShapeError(f"head_dim must be 16, 32, 64 or 128, got {q.shape[-1]}")
     if not (q.device == k.device == v.device):
         raise ShapeError("q, k, v must be on the same device")
 
@@ -162,7 +183,7 @@ def _dense_launch(q, k, v, scale, want_o=True, want_ml=True, want_lse2=False):
     with _on_device(q):
         stream = _stream(q)
         st = _lib.load().lvar_dense_attn_ws_fwd(_view(q), _view(k), _view(v if want_o else None), _view(o), _ptr(M), _ptr(L),
-                                               _ptr(lse2), B, H, Lq, Lk, d, _scale(q, scale),
+                                               _ptr(lse2), B, H, k.shape[1], Lq, Lk, d, _scale(q, scale),
                                                _workspace(q, stream) if want_o else _NO_WORKSPACE, stream)
     _lib.check(st, "lvar_dense_attn_ws_fwd")
     return o, M, L, lse2
@@ -177,10 +198,13 @@ def dense_attn(q, k, v, scale=None):
         r = fast.fast_dense_attn(q, k, v, None if scale is None else float(scale)) if isinstance(q, torch.Tensor) else None
         if r is not None:
             return r[0], (r[1], r[2])
+    q, k, v, d_small = _pad_head_dim(q, k, v)
+    if d_small is not None:
+        scale = _scale_for(d_small, scale)
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
-    _check_qkv(q, k, v)
+    _check_qkv(q, k, v, gqa=True)
     o, M, L, _ = _dense_launch(q, k, v, scale)
-    return o, (M, L)
+    return (o if d_small is None else o[..., :d_small].contiguous()), (M, L)
 
 
 def _lse_only(q, k, scale):
@@ -196,7 +220,7 @@ def _colsum_given_lse(q, k, lse2, scale, q_group_size, want_block_sums=False):
     bs = torch.empty((B, H, G, (Lk + 63) // 64), dtype=torch.float32, device=q.device) if want_block_sums else None
     with _on_device(q):
         st = _lib.load().lvar_colsum_fwd(_view(q), _view(k), lse2.data_ptr(), cs.data_ptr(), _ptr(bs),
-                                        B, H, Lq, Lk, d, q_group_size, _scale(q, scale), _stream(q))
+                                        B, H, k.shape[1], Lq, Lk, d, q_group_size, _scale(q, scale), _stream(q))
     _lib.check(st, "lvar_colsum_fwd")
     return (cs, bs) if want_block_sums else cs
 
@@ -207,8 +231,11 @@ def colsum(q, k, scale=None, q_group_size: Optional[int] = None, lse: Optional[T
     (default: the kernel config's ``bm`` = 192), fp32 ``[B,H,G,Lk]``.  Self-contained two-pass form
     (statistics sweep, then column sweep) unless ``lse=(M, L)`` from a previous dense pass is given.
     With ``return_block_sums`` also returns the sums over blocks of 64 keys, ``[B,H,G,ceil(Lk/64)]``."""
+    q, k, _, d_small = _pad_head_dim(q, k)
+    if d_small is not None:
+        scale = _scale_for(d_small, scale)
     q, k = _prep(q, "q"), _prep(k, "k")
-    _check_qkv(q, k, k)
+    _check_qkv(q, k, k, gqa=True)
     if q_group_size is None:
         q_group_size = get_kernel_config_attn()["bm"]
     _require(q_group_size > 0 and q_group_size % 32 == 0, "q_group_size must be a positive multiple of 32")
@@ -225,11 +252,14 @@ def dense_colsum_attn(q, k, v, scale=None):
     """Kernel-level op ``(o, blocksums, (M, L))`` (reference Triton ``dense_colsum_attn``,
     kernels/sparse_attn/triton/attn_dense_colsum.py:237-296): dense attention, then the column
     sweep that reuses its row statistics."""
+    q, k, v, d_small = _pad_head_dim(q, k, v)
+    if d_small is not None:
+        scale = _scale_for(d_small, scale)
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
-    _check_qkv(q, k, v)
+    _check_qkv(q, k, v, gqa=True)
     o, M, L, lse2 = _dense_launch(q, k, v, scale, want_lse2=True)
     cs = _colsum_given_lse(q, k, lse2, scale, get_kernel_config_attn()["bm"])
-    return o, cs, (M, L)
+    return (o if d_small is None else o[..., :d_small].contiguous()), cs, (M, L)
 
 
 def dense_colsum_attn_s(q, k, v, scale=None):
@@ -250,6 +280,15 @@ def dense_colsum_attn_q(q, k, v, scale=None):
 
 
 def _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, upsample_from=None, out=None):
+    q, k, v, d_small = _pad_head_dim(q, k, v)
+    if d_small is not None:
+        if out is not None:
+            raise ShapeError("the in-place op needs head_dim 64 or 128")
+        scale = _scale_for(d_small, scale)
+        if o_accum is not None:
+            o_accum = torch.nn.functional.pad(o_accum, (0, 64 - d_small))
+        res = _csp_launch(q, k, v, indices, counts, o_accum, o_scale, scale, want_stats, upsample_from)
+        return (res[0][..., :d_small].contiguous(),) + tuple(res[1:])
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
     _check_qkv(q, k, v)
     B, H, Lq, d = q.shape
@@ -337,6 +376,10 @@ def block_sparse_attn(q, k, v, kv_num_blocks, kv_indices, block_q: int = 128, bl
     ``BlockMask`` layout consumed by ``SparseFlexAttn`` (models/sparvar/basic_sparvar.py:55-72,187-194):
     ``kv_num_blocks`` int32 ``[B|1,H|1,nQ]``, ``kv_indices`` int32 ``[B|1,H|1,nQ,nKmax]``.
     Returns ``(o, (M, L))``."""
+    q, k, v, d_small = _pad_head_dim(q, k, v)
+    if d_small is not None:
+        o, ml = block_sparse_attn(q, k, v, kv_num_blocks, kv_indices, block_q, block_k, _scale_for(d_small, scale))
+        return o[..., :d_small].contiguous(), ml
     q, k, v = _prep(q, "q"), _prep(k, "k"), _prep(v, "v")
     _check_qkv(q, k, v)
     B, H, Lq, d = q.shape

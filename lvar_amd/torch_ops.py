@@ -36,20 +36,20 @@ _registered = {}      # namespace -> the torch.library.Library objects that keep
 
 def _dense_attn(q, k, v):
     q, k, v = ops._prep(q, "q"), ops._prep(k, "k"), ops._prep(v, "v")
-    ops._check_qkv(q, k, v)
+    ops._check_qkv(q, k, v, gqa=True)
     B, H, Lq, d = q.shape
     o = torch.empty_like(q)
     rcp = torch.empty((B, H, Lq, 1), dtype=torch.float32, device=q.device)
     with ops._on_device(q):
         st = _lib.load().lvar_dense_attn_rcp_fwd(ops._view(q), ops._view(k), ops._view(v), ops._view(o), rcp.data_ptr(),
-                                                B, H, Lq, k.shape[2], d, 1.0, ops._stream(q))
+                                                B, H, k.shape[1], Lq, k.shape[2], d, 1.0, ops._stream(q))
     _lib.check(st, "lvar_dense_attn_rcp_fwd")
     return [o, rcp]
 
 
 def _dense_colsum_attn(q, k, v, p):
     q, k, v = ops._prep(q, "q"), ops._prep(k, "k"), ops._prep(v, "v")
-    ops._check_qkv(q, k, v)
+    ops._check_qkv(q, k, v, gqa=True)                    # dense_colsum_attn.cu:386-387
     if tuple(p.shape) != (q.shape[0], q.shape[1], q.shape[2], 1):
         raise ops.ShapeError(f"P shape mismatch - p: {tuple(p.shape)}, q: {tuple(q.shape)}")
     o, _, _, lse2 = ops._dense_launch(q, k, v, 1.0, want_ml=False, want_lse2=True)

@@ -29,7 +29,7 @@ __all__ = [
     "aggregate_group_indices", "upsample_ocache", "flex_block_mask", "infinity_cum",
     "INFINITY_SCALES", "config2_block_mask", "attn_flops_blocks", "attn_flops_lists",
     "topk_token_set", "append_local_run", "mask_to_lists", "window_key_scores",
-    "video_window_block_mask", "base_plus_topk_block_mask",
+    "video_window_block_mask", "base_plus_topk_block_mask", "expand_kv_heads",
 ]
 
 # Infinity "1M" scale schedule, reference utils/dynamic_resolution.py:7 and
@@ -547,3 +547,14 @@ def base_plus_topk_block_mask(block_scores, base, target):
                 order = cand[np.argsort(-sc[b, h, i, cand], kind="stable")]
                 out[b, h, i, order[:extra]] = True
     return torch.from_numpy(out)
+
+
+def expand_kv_heads(k, qo_heads):
+    """Grouped-query attention: K or V with ``kv_heads`` heads broadcast to ``qo_heads`` query heads, query head
+    ``h`` reading K/V head ``h // (qo_heads // kv_heads)`` (kernels/sparse_attn/sparse_attn_ops.py:228-233:
+    ``unsqueeze(2).expand(B, kv_h, hr, L, d).reshape(B, qo_h, L, d)``; kernels/chipmunk/csrc/attn/
+    dense_colsum_attn.cu:106 ``kv_head_idx = blockIdx.y / hr``)."""
+    B, kv_h, L, d = k.shape
+    assert qo_heads % kv_h == 0, "qo_heads must be a multiple of kv_heads"
+    hr = qo_heads // kv_h
+    return k.unsqueeze(2).expand(B, kv_h, hr, L, d).reshape(B, qo_heads, L, d)

@@ -47,16 +47,18 @@ def test_argument_validation_without_device(lib):
     fake = LvarTensor(0x1000, 128 * 16 * 128, 16 * 128, 128)          # aligned, never dereferenced
     odd = LvarTensor(0x1008, 128 * 16 * 128, 16 * 128, 128)           # misaligned base
     one = ctypes.c_void_p(0x2000)
-    assert lib.lvar_dense_attn_fwd(null, fake, fake, fake, one, one, None, 1, 1, 16, 16, 128, 1.0, None) == -1
-    assert lib.lvar_dense_attn_fwd(odd, fake, fake, fake, one, one, None, 1, 1, 16, 16, 128, 1.0, None) == -1
-    assert lib.lvar_dense_attn_fwd(fake, fake, fake, fake, one, one, None, 0, 1, 16, 16, 128, 1.0, None) == -1
-    assert lib.lvar_dense_attn_fwd(fake, fake, fake, fake, one, one, None, 1, 1, 16, 16, 128, -1.0, None) == -1
-    assert lib.lvar_dense_attn_fwd(fake, fake, null, null, None, None, None, 1, 1, 16, 16, 128, 1.0, None) == -1   # no outputs at all
-    assert lib.lvar_colsum_fwd(fake, fake, one, one, None, 1, 1, 16, 16, 128, 100, 1.0, None) == -1           # group not a multiple of 32
-    assert lib.lvar_colsum_fwd(fake, fake, None, one, None, 1, 1, 16, 16, 128, 192, 1.0, None) == -1
+    assert lib.lvar_dense_attn_fwd(null, fake, fake, fake, one, one, None, 1, 1, 1, 16, 16, 128, 1.0, None) == -1
+    assert lib.lvar_dense_attn_fwd(odd, fake, fake, fake, one, one, None, 1, 1, 1, 16, 16, 128, 1.0, None) == -1
+    assert lib.lvar_dense_attn_fwd(fake, fake, fake, fake, one, one, None, 0, 1, 1, 16, 16, 128, 1.0, None) == -1
+    assert lib.lvar_dense_attn_fwd(fake, fake, fake, fake, one, one, None, 1, 1, 1, 16, 16, 128, -1.0, None) == -1
+    assert lib.lvar_dense_attn_fwd(fake, fake, null, null, None, None, None, 1, 1, 1, 16, 16, 128, 1.0, None) == -1   # no outputs at all
+    assert lib.lvar_dense_attn_fwd(fake, fake, fake, fake, one, one, None, 1, 6, 4, 16, 16, 128, 1.0, None) == -1   # 6 query heads over 4 K/V heads
+    assert lib.lvar_colsum_fwd(fake, fake, one, one, None, 1, 6, 0, 16, 16, 128, 192, 1.0, None) == -1
+    assert lib.lvar_colsum_fwd(fake, fake, one, one, None, 1, 1, 1, 16, 16, 128, 100, 1.0, None) == -1           # group not a multiple of 32
+    assert lib.lvar_colsum_fwd(fake, fake, None, one, None, 1, 1, 1, 16, 16, 128, 192, 1.0, None) == -1
     assert lib.lvar_csp_attn_fwd(fake, fake, fake, null, fake, None, None, one, one, 1, 16, 100, 1, 1, 16, 16, 128, 1.0, 1.0, None) == -2   # groups of 100 rows: no workgroup shape
     assert lib.lvar_csp_attn_fwd(fake, fake, fake, null, fake, None, None, one, one, 1, 16, 0, 1, 1, 16, 16, 128, 1.0, 1.0, None) == -1
-    assert lib.lvar_dense_attn_rcp_fwd(fake, fake, fake, fake, None, 1, 1, 16, 16, 128, 1.0, None) == -1                # no place for the row constant
+    assert lib.lvar_dense_attn_rcp_fwd(fake, fake, fake, fake, None, 1, 1, 1, 16, 16, 128, 1.0, None) == -1                # no place for the row constant
     assert lib.lvar_csp_attn_fwd(fake, fake, fake, null, fake, None, None, None, one, 1, 16, 192, 1, 1, 16, 16, 128, 1.0, 1.0, None) == -1
     assert lib.lvar_block_sparse_attn_fwd(fake, fake, fake, fake, None, None, one, 0, 0, one, 0, 0, 4, 4, 64, 64, 1, 1, 16, 16, 128, 1.0, None) == -2
     wide = LvarTensor(0x1000, 1 << 30, 1 << 26, 1 << 23)                # row stride of 2^23 elements: beyond the 24-bit gather addressing

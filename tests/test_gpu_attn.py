@@ -308,6 +308,61 @@ def test_errors():
                      torch.zeros(1, 1, 1, dtype=torch.int32).cuda(), qg, 1)
     with pytest.raises(RuntimeError):
         ops.dense_attn(q, k, v)  # CPU tensors: no fallback
-    q32, k32, v32 = make_qkv(1, 1, 64, 64, 32, seed=1)
+    q48, k48, v48 = make_qkv(1, 1, 64, 64, 48, seed=1)
     with pytest.raises(AssertionError):
-        ops.dense_attn(*dev(q32, k32, v32))
+        ops.dense_attn(*dev(q48, k48, v48))      # head_dim 48: neither a kernel width nor padded to one
+
+
+@pytest.mark.parametrize("H,Hkv", [(8, 2), (6, 1), (4, 4)])
+def test_grouped_query_attention(H, Hkv):
+    """Fewer K/V heads than query heads (dense_colsum_attn.cu:386-387; sparse_attn_ops.py:228-233): query head h
+    reads K/V head h // (H // Hkv); dense attention, colsum (per query head) and the fused pair, through the operator
+    API and the torch-library op."""
+    import lvar_amd.torch_ops  # noqa: F401
+    from lvar_amd import sparse_attn_ops as ops
+    B, Lq, Lk, d = 2, 400, 777, 128
+    q, _, _ = make_qkv(B, H, Lq, Lk, d, seed=H * 10 + Hkv, amp=0.7)
+    _, k, v = make_qkv(B, Hkv, Lq, Lk, d, seed=H * 10 + Hkv + 1, amp=0.7)
+    ke, ve = oracle.expand_kv_heads(k, H), oracle.expand_kv_heads(v, H)
+    o_ref, cs_ref, (M_ref, L_ref) = oracle.dense_colsum_attn(q, ke, ve)[0], oracle.dense_colsum_attn(q, ke, ve)[1], oracle.dense_attn(q, ke, ve)[1:]
+    qg, kg, vg = dev(q, k, v)
+    o, (M, L) = ops.dense_attn(qg, kg, vg)
+    check_o(o, o_ref, "gqa dense")
+    check_lse(M, L, M_ref, L_ref)
+    o2, cs, _ = ops.dense_colsum_attn(qg, kg, vg)
+    assert torch.equal(o2, o) and cs.shape == (B, H, 3, Lk)
+    assert torch.allclose(cs.cpu(), cs_ref, rtol=1e-3, atol=1e-6)
+    assert torch.allclose(ops.colsum(qg, kg).cpu(), cs_ref, rtol=1e-3, atol=1e-6)
+    o3, lse = torch.ops.lvar.dense_attn(qg, kg, vg)
+    check_o(o3, oracle.dense_attn(q, ke, ve, scale=1.0)[0], "gqa torch op")
+    if H != Hkv:
+        with pytest.raises(AssertionError):
+            ops.block_sparse_attn(qg, kg, vg, torch.ones(1, 1, 4, dtype=torch.int32).cuda(), torch.zeros(1, 1, 4, 13, dtype=torch.int32).cuda())
+        with pytest.raises(AssertionError):
+            ops.dense_attn(qg, kg[:, :0], vg[:, :0])
+
+
+@pytest.mark.parametrize("d", [16, 32])
+def test_small_head_dims_by_zero_padding(d):
+    """head_dim 16 and 32 (attn_dense_colsum.py:246 takes them) run on the 64-wide kernels with zero columns."""
+    from lvar_amd import mask_build as mb, sparse_attn_ops as ops
+    B, H, Lq, Lk = 1, 3, 300, 450
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=d, amp=1.0)
+    qg, kg, vg = dev(q, k, v)
+    o_ref, M_ref, L_ref = oracle.dense_attn(q, k, v)
+    o, (M, L) = ops.dense_attn(qg, kg, vg)
+    assert o.shape == q.shape
+    check_o(o, o_ref, f"d={d}")
+    check_lse(M, L, M_ref, L_ref)
+    o2, cs, _ = ops.dense_colsum_attn(qg, kg, vg)
+    _, cs_ref, _ = oracle.dense_colsum_attn(q, k, v)
+    assert torch.equal(o2, o) and torch.allclose(cs.cpu(), cs_ref, rtol=1e-3, atol=1e-6)
+    inds, counts = mb.topk_index_list(cs, 0.3)
+    out = ops.csp_attn(qg, kg, vg, 0.3, inds, counts, o, -1)
+    check_o(out, oracle.csp_attn(q, k, v, 0.3, inds.cpu(), counts.cpu(), o.cpu(), -1), "csp small d")
+    mask = torch.rand(B, H, 3, (Lk + 63) // 64, generator=torch.Generator().manual_seed(d)) < 0.5
+    num, idx = oracle.block_mask_to_lists(mask)
+    ob, _ = ops.block_sparse_attn(qg, kg, vg, num.cuda(), idx.cuda(), 128, 64)
+    check_o(ob, oracle.block_sparse_attn(q, k, v, num, idx, 128, 64)[0], "block small d")
+    with pytest.raises(AssertionError):
+        ops.dense_attn(*dev(*make_qkv(1, 1, 8, 8, 256, seed=1)))

@@ -222,7 +222,7 @@ def test_small_workspace_and_plain_fallback(ops):
         M = torch.empty(B, H, Lq, 1, dtype=torch.float32, device="cuda")
         L = torch.empty_like(M)
         st = lib.lvar_dense_attn_ws_fwd(ops._view(qg), ops._view(kg), ops._view(vg), ops._view(o), M.data_ptr(), L.data_ptr(), None,
-                                        B, H, Lq, Lk, d, 1.0 / d ** 0.5, ws, ops._stream(qg))
+                                        B, H, H, Lq, Lk, d, 1.0 / d ** 0.5, ws, ops._stream(qg))
         assert st == 0 and close(o, o_ref)
         if want == 0:
             assert torch.equal(o, o_plain) and torch.equal(M, M_plain) and torch.equal(L, L_plain)
@@ -235,7 +235,7 @@ def test_small_workspace_and_plain_fallback(ops):
     ws = _lib.LvarWorkspace(buf.data_ptr() + 16, full, 0, 0)
     o = torch.empty_like(qg)
     assert lib.lvar_dense_attn_ws_fwd(ops._view(qg), ops._view(kg), ops._view(vg), ops._view(o), None, None, None,
-                                      B, H, Lq, Lk, d, 1.0 / d ** 0.5, ws, ops._stream(qg)) == -1
+                                      B, H, H, Lq, Lk, d, 1.0 / d ** 0.5, ws, ops._stream(qg)) == -1
 
 
 def test_balanced_share_and_piece_knobs(ops):

@@ -381,3 +381,12 @@ def test_window_key_scores_bruteforce():
                 exp = -math.inf if n in wk else (sum(nb) / ks if pooling == "avgpool" else max(nb))
                 g = float(got[0, h, n])
                 assert (g == exp) if math.isinf(exp) else abs(g - exp) < 1e-9, (pooling, h, n, g, exp)
+
+
+def test_expand_kv_heads_matches_repeat_interleave():
+    k = rnd(2, 3, 5, 4, seed=1)
+    e = oracle.expand_kv_heads(k, 12)
+    assert e.shape == (2, 12, 5, 4) and torch.equal(e, k.repeat_interleave(4, dim=1))
+    for h in range(12):
+        assert torch.equal(e[:, h], k[:, h // 4])
+    assert torch.equal(oracle.expand_kv_heads(k, 3), k)
