@@ -28,18 +28,43 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X published dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel
-# of known size; the summaries are under profiles/.  None = not measured for that workload.
-MEASURED_TRAFFIC = {
-    # profiles/attn_fwd_block_sparse_infinity2b_1024_last_scale_25pct.txt: FETCH 100990 KiB x 2.0 + WRITE 33741 KiB x 1.0
-    "block_sparse_25": 241.4e6,
-    # profiles/attn_fwd_dense_infinity2b_1024_last_scale.txt: FETCH 100700 KiB x 2.0 + WRITE 33792 KiB x 1.0
-    "dense": 240.8e6,
-    # profiles/colsum_infinity2b_1024_last_scale.txt: FETCH 65760 KiB x 2.0 + WRITE 28990 KiB x 1.0
-    "colsum": 164.4e6,
-    # profiles/attn_fwd_token_list_infinity2b_1024_last_scale_top20pct.txt: FETCH 141270 KiB x 2.0 + WRITE 32717 KiB x 1.0
-    "csp": 322.8e6,
+# HBM bytes per launch are measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known
+# size, and recorded in the summary under profiles/ that covers the workload, as the line
+#   traffic_bytes_per_launch: <bytes>
+# next to the SHA-256 of the kernel source the measurement was taken with:
+#   kernel_source_sha256: <file under lvar_amd/csrc> <hex digest>
+# The bench line carries the figure only while that source file is unchanged.
+PROFILE_OF_WORKLOAD = {
+    "block_sparse_25": "attn_fwd_block_sparse_infinity2b_1024_last_scale_25pct.txt",
+    "dense": "attn_fwd_dense_infinity2b_1024_last_scale.txt",
+    "colsum": "colsum_infinity2b_1024_last_scale.txt",
+    "csp": "attn_fwd_token_list_infinity2b_1024_last_scale_top20pct.txt",
 }
+
+
+def measured_traffic(workload):
+    """(bytes per launch or None, where it comes from / why it is missing)."""
+    import hashlib
+    import re
+    name = PROFILE_OF_WORKLOAD.get(workload)
+    if name is None:
+        return None, "no counter profile for this workload"
+    path = os.path.join(ROOT, "profiles", name)
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, f"profiles/{name} is missing"
+    m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, re.M)
+    h = re.search(r"^kernel_source_sha256:\s*(\S+)\s+([0-9a-f]{64})", text, re.M)
+    if not m or not h:
+        return None, f"profiles/{name} records no traffic figure"
+    try:
+        digest = hashlib.sha256(open(os.path.join(ROOT, "lvar_amd", "csrc", h.group(1)), "rb").read()).hexdigest()
+    except OSError:
+        return None, f"lvar_amd/csrc/{h.group(1)} is missing"
+    if digest != h.group(2):
+        return None, f"lvar_amd/csrc/{h.group(1)} has changed since profiles/{name} was taken"
+    return float(m.group(1)), f"profiles/{name}"
 
 
 def make_qkv(B, H, Lq, Lk, d, seed, amp):
@@ -336,7 +361,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="block_sparse_25",
-                    help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | density_<pct> | video_10 | infinity2b_schedule | topk_tokens | remap_lists | window_scores | copy_1gib")
+                    help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | full_step | density_<pct> | video_10 | infinity2b_schedule | topk_tokens | remap_lists | window_scores | copy_1gib")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aux", action="store_true", help="skip the companion dense/colsum/mask-build timings")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0)
@@ -384,6 +409,8 @@ def main():
         amp = 1.0 if (wl.startswith("density_") or wl == "colsum") else 0.5
     elif wl == "colsum_scale48":
         B, H, Lq, Lk, amp = 2, 16, 2304, 6425, 1.0
+    elif wl == "full_step":
+        B, H, Lq, Lk, amp = 2, 16, 1600, 4121, 0.5
     elif wl == "video_10":
         B, H, Lq, Lk, amp = 1, 24, 32768, 32768, 0.5
     else:
@@ -444,6 +471,28 @@ def main():
             done, t = cpu_baseline_dense(q, k, v, args.cpu_budget_s, colsum=True)
             cpu = {"value": round(1.5 * dense_flops / (B * H) * done / t / 1e12, 5), "unit": "TFLOP/s", "cores": os.cpu_count(),
                    "kind": "port", "sample": f"{done} (batch,head) slices (the workload has {B * H}; cycled) of dense attention + colsum (6*Lq*Lk*d flops each), {t:.1f} s of host time"}
+    elif wl == "full_step":
+        # decision-scale step of the CS4A caller (models/sparvar/sparse_attn.py:1006-1049): dense attention + colsum +
+        # top-k key lists + O_cache = O - delta over the selected keys; effective rate over the dense flops
+        from lvar_amd import sparse_attn_config as cfgmod
+        from lvar_amd.sparse_diff_attn import SparseDiffAttn
+        cfgmod.reset()
+        cfgmod.GLOBAL_CONFIG["attn"]["top_keys"] = 0.2
+        mod = SparseDiffAttn(0, None, spsd_scale=10)
+        flops = dense_flops
+        fn = lambda: mod(qg, kg, vg, scale, do_full_step=True, scale_ind=10)
+        kernel = "attn_fwd_kernel<128,4,MODE_BLOCK> + colsum_kernel<128> + topk_token_lists_kernel + attn_fwd_kernel<128,8,MODE_GATHER>"
+        dense_ms, _ = time_launches(lambda: ops.dense_attn(qg, kg, vg, scale), 20, 5)
+        lse2 = ops._lse_only(qg, kg, scale)
+        o_d, _, _, _ = ops._dense_launch(qg, kg, vg, scale)
+        cs = ops._colsum_given_lse(qg, kg, lse2, scale, 192)
+        i_d, c_d = mb.topk_index_list(cs, 0.2, order="index")
+        parts = {"dense_attn_us": dense_ms * 1e3,
+                 "colsum_us": time_launches(lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 192), 20, 5)[0] * 1e3,
+                 "topk_lists_us": time_launches(lambda: mb.topk_index_list(cs, 0.2, order="index"), 20, 5)[0] * 1e3,
+                 "ocache_csp_us": time_launches(lambda: ops.csp_attn(qg, kg, vg, scale, i_d, c_d, o_d, -1), 20, 5)[0] * 1e3}
+        aux = {k_: round(v_, 1) for k_, v_ in parts.items()}
+        config.update({"top_keys": 0.2, "decision_scale": 10, "count": int(c_d[0, 0, 0])})
     elif wl == "csp":
         G = (Lq + 191) // 192
         cs = ops.colsum(qg, kg, scale)
@@ -487,6 +536,11 @@ def main():
                "colsum_given_lse_us": round(cs_ms * 1e3, 1), "lse_pass_us": round(lse_ms * 1e3, 1),
                "colsum_plus_mask_build_ms": round(build_ms, 4), "speedup_vs_dense": round(dense_ms / ms, 3)}
 
+    traffic, traffic_src = measured_traffic(wl)
+    dev_sum = device_summary()
+    # CU count x 4096 flop per clock x maximum engine clock, as the device reports them at run time; `peak` and
+    # `frac` stay the published 2.5 PFLOP/s
+    peak_rt = dev_sum.get("bf16_mfma_tflops_from_cus_and_clock")
     out = {
         "metric": ("block-sparse attn effective TFLOP/s (% bf16 MFMA peak); colsum us @Infinity-2B 1024^2"
                    if wl == "block_sparse_25" else f"{wl} effective TFLOP/s"),
@@ -495,13 +549,17 @@ def main():
         "dtype": "bf16", "data": "synthetic (seeded N(0,1)*%.1f, random-init, no checkpoint)" % amp,
         "config": config,
         "roofline": {"bound": "mfma", "kernel": kernel, "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC.get(wl),
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": traffic, "traffic_source": traffic_src,
+                     "peak_runtime": peak_rt, "frac_runtime": (round(tflops / peak_rt, 4) if peak_rt else None),
                      "flops_per_launch": flops, "host_wall_ms_per_step": round(wall_ms, 5),
                      "single_launch": single, "cache_state": "warm: back-to-back launches on the same inputs, no L2 flush",
                      "settle_ms": SETTLE_MS},
         "cpu_baseline": cpu,
-        "device": torch.cuda.get_device_name(0), "device_summary": device_summary(),
+        "device": torch.cuda.get_device_name(0), "device_summary": dev_sum,
     }
+    if wl == "full_step":
+        aux["full_step_us"] = round(ms * 1e3, 1)
+        aux["full_step_over_dense"] = round(ms / dense_ms, 3)
     if aux:
         out["aux"] = aux
     print(json.dumps(out))
