@@ -288,7 +288,7 @@ def run_hbm_workload(args, dev, wl):
         cs = cs_cpu.to(dev)
         idx = torch.zeros(B, H, G, Lk, dtype=torch.int32, device=dev)
         cn = torch.empty(B, H, G, dtype=torch.int32, device=dev)
-        fn = lambda: lib.lvar_topk_token_lists(cs.data_ptr(), Lk, idx.data_ptr(), Lk, cn.data_ptr(), B * H * G, Lk, cnt, stream)
+        fn = lambda: lib.lvar_topk_token_lists(cs.data_ptr(), Lk, idx.data_ptr(), Lk, cn.data_ptr(), B * H * G, Lk, cnt, 0, stream)
         nbytes = B * H * G * (Lk * 4 + cnt * 4 + 4)
         kernel, unit_desc = "topk_token_lists_kernel<24,512>", f"{B * H * G} rows x {Lk} fp32 scores, k = {cnt}"
         fn()
@@ -309,7 +309,7 @@ def run_hbm_workload(args, dev, wl):
         out = torch.zeros(B, H, G, Lk, dtype=torch.int32, device=dev)
         cn = torch.empty(B, H, G, dtype=torch.int32, device=dev)
         fn = lambda: lib.lvar_remap_concat_lists(src.data_ptr(), Ks, Ks, loc.data_ptr(), L, L, out.data_ptr(), Lk, cn.data_ptr(),
-                                                 B * H, Gs, G, cnt, Lk, stream)
+                                                 B * H, Gs, G, cnt, Lk, 0, stream)
         nbytes = B * H * G * ((cnt + L) * 4 + cnt * 4 + L * 8 + 4)
         kernel, unit_desc = "remap_concat_lists_kernel", f"{B * H * G} output rows: {cnt} remapped + {L} local keys"
         if not args.no_cpu_baseline:

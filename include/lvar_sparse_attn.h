@@ -256,7 +256,8 @@ int lvar_block_topk_lists(const float* block_scores, const uint8_t* base_mask,
  * Exact top-k key selection per row: for each of `rows` rows of `scores` (fp32, row stride
  * score_row_stride >= Lk elements; e.g. the [B*H*G, Lk] view of the column sums) write the columns
  * of the k largest values, in ASCENDING column order, to indices[row, 0:k] (row stride
- * idx_row_stride >= k; columns >= k are left untouched) and, if counts is not NULL, k to counts[row].
+ * idx_row_stride >= k; columns [k, zero_to) are set to 0, zero_to <= idx_row_stride, the rest is left untouched)
+ * and, if counts is not NULL, k to counts[row].
  * Ties at the k-th value go to the smaller column, so the selected SET equals that of a stable
  * descending sort and is a pure function of the scores.  Radix select, no sort: the rows are read
  * five times from L2.  Replaces `torch.topk(bs, k=indices_count, dim=-1).indices` of the full step
@@ -265,7 +266,7 @@ int lvar_block_topk_lists(const float* block_scores, const uint8_t* base_mask,
  */
 int lvar_topk_token_lists(const float* scores, int64_t score_row_stride,
                           int32_t* indices, int64_t idx_row_stride, int32_t* counts,
-                          int rows, int Lk, int k, void* stream);
+                          int rows, int Lk, int k, int zero_to, void* stream);
 
 /*
  * Sparse-step key list in one launch: for every (batch*head) slice bh < BH and query group g < Gk of
@@ -276,14 +277,15 @@ int lvar_topk_token_lists(const float* scores, int64_t score_row_stride,
  * where gS(g) = clamp(rint((g + 0.5) / Gk * Gs - 0.5), 0, Gs-1) in fp32 with round-half-to-even,
  * rep = 1 if src_len >= count else ceil(count / src_len).  src_indices is int32 [BH, Gs, src_row_stride]
  * (first src_len columns valid), local_indices int64 [Gk, local_row_stride] (may be NULL with
- * local_count = 0), out_indices int32 [BH*Gk, out_row_stride >= count + local_count].
+ * local_count = 0), out_indices int32 [BH*Gk, out_row_stride >= count + local_count]; columns
+ * [count + local_count, zero_to) of every output row are set to 0 (zero_to <= out_row_stride, 0 = untouched).
  * Replaces map_inds_counts_across_scales (models/sparvar/sparse_attn.py:366-421) followed by the
  * top-k-then-local concatenation and padding of the sparse step (models/sparvar/sparse_attn.py:1096-1121).
  */
 int lvar_remap_concat_lists(const int32_t* src_indices, int64_t src_row_stride, int src_len,
                             const int64_t* local_indices, int64_t local_row_stride, int local_count,
                             int32_t* out_indices, int64_t out_row_stride, int32_t* out_counts,
-                            int BH, int Gs, int Gk, int count, int Lk, void* stream);
+                            int BH, int Gs, int Gk, int count, int Lk, int zero_to, void* stream);
 
 /*
  * Mask compaction: for each of `rows` rows of a uint8 mask (row stride mask_row_stride >= n) write the

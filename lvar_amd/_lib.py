@@ -85,9 +85,9 @@ def load() -> C.CDLL:
     lib.lvar_block_topk_lists.restype = I
     lib.lvar_block_topk_lists.argtypes = [P, P, P, P, I, I, I, I, I, P]
     lib.lvar_topk_token_lists.restype = I
-    lib.lvar_topk_token_lists.argtypes = [P, I64, P, I64, P, I, I, I, P]
+    lib.lvar_topk_token_lists.argtypes = [P, I64, P, I64, P, I, I, I, I, P]
     lib.lvar_remap_concat_lists.restype = I
-    lib.lvar_remap_concat_lists.argtypes = [P, I64, I, P, I64, I, P, I64, P, I, I, I, I, I, P]
+    lib.lvar_remap_concat_lists.argtypes = [P, I64, I, P, I64, I, P, I64, P, I, I, I, I, I, I, P]
     lib.lvar_mask_to_lists.restype = I
     lib.lvar_mask_to_lists.argtypes = [P, I64, P, I64, P, I, I, I, P]
     lib.lvar_window_key_scores.restype = I

@@ -332,28 +332,29 @@ int lvar_block_topk_lists(const float* block_scores, const uint8_t* base_mask, i
 }
 
 int lvar_topk_token_lists(const float* scores, int64_t score_row_stride, int32_t* indices, int64_t idx_row_stride,
-                          int32_t* counts, int rows, int Lk, int k, void* stream) {
-  if (!scores || !indices || rows < 0 || Lk <= 0 || k < 0 || k > Lk || score_row_stride < Lk || idx_row_stride < k)
+                          int32_t* counts, int rows, int Lk, int k, int zero_to, void* stream) {
+  if (!scores || !indices || rows < 0 || Lk <= 0 || k < 0 || k > Lk || score_row_stride < Lk || idx_row_stride < k ||
+      zero_to < 0 || zero_to > idx_row_stride)
     return LVAR_EINVAL;
   TopkListParams p{};
   p.scores = scores; p.indices = indices; p.counts = counts;
   p.score_stride = score_row_stride; p.out_stride = idx_row_stride;
-  p.rows = rows; p.n = Lk; p.k = k;
+  p.rows = rows; p.n = Lk; p.k = k; p.zero_to = zero_to;
   return launch_topk_token_lists(p, (hipStream_t)stream);
 }
 
 int lvar_remap_concat_lists(const int32_t* src_indices, int64_t src_row_stride, int src_len,
                             const int64_t* local_indices, int64_t local_row_stride, int local_count,
                             int32_t* out_indices, int64_t out_row_stride, int32_t* out_counts,
-                            int BH, int Gs, int Gk, int count, int Lk, void* stream) {
+                            int BH, int Gs, int Gk, int count, int Lk, int zero_to, void* stream) {
   if (!src_indices || !out_indices || BH < 0 || Gs <= 0 || Gk <= 0 || count < 0 || Lk <= 0 || src_len <= 0 ||
       src_row_stride < src_len || local_count < 0 || (local_count > 0 && (!local_indices || local_row_stride < local_count)) ||
-      out_row_stride < (int64_t)count + local_count)
+      out_row_stride < (int64_t)count + local_count || zero_to < 0 || zero_to > out_row_stride)
     return LVAR_EINVAL;
   RemapListParams p{};
   p.src = src_indices; p.local = local_count > 0 ? local_indices : nullptr; p.out = out_indices; p.counts = out_counts;
   p.src_stride = src_row_stride; p.local_stride = local_row_stride; p.out_stride = out_row_stride;
-  p.rows = BH * Gk; p.Gs = Gs; p.Gk = Gk; p.cnt = count; p.L = local_count; p.Lk = Lk;
+  p.rows = BH * Gk; p.Gs = Gs; p.Gk = Gk; p.cnt = count; p.L = local_count; p.Lk = Lk; p.zero_to = zero_to;
   p.rep = (src_len >= count) ? 1 : (count + src_len - 1) / src_len;
   return launch_remap_concat_lists(p, (hipStream_t)stream);
 }

@@ -79,6 +79,7 @@ struct TopkListParams {
   int32_t* counts;      // [rows] or null
   int64_t score_stride, out_stride;
   int rows, n, k;
+  int zero_to;          // columns [k, zero_to) of every index row are set to 0 (0 = left untouched)
 };
 
 struct RemapListParams {
@@ -88,6 +89,7 @@ struct RemapListParams {
   int32_t* counts;       // [BH*Gk] or null
   int64_t src_stride, local_stride, out_stride;
   int rows, Gs, Gk, cnt, rep, L, Lk;
+  int zero_to;           // columns [cnt + L, zero_to) of every output row are set to 0 (0 = left untouched)
 };
 
 struct MaskCompactParams {

@@ -43,6 +43,8 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
   const int n = p.n;
   int want = min(max(p.k, 0), n);  // keys still to be found among those matching the prefix
   if (tid == 0 && p.counts) p.counts[row] = want;
+  // columns [k, zero_to) of the list row: defined (zero) instead of whatever the buffer held
+  for (int t = want + tid; t < p.zero_to; t += NT) out[t] = 0;
   if (want == 0) return;
 
   // chunk c of wave w covers columns (w * cpw + c) * 64 .. +63
@@ -172,7 +174,9 @@ __global__ __launch_bounds__(256) void remap_concat_lists_kernel(const RemapList
     const int64_t* loc = p.local + (int64_t)g * p.local_stride;
     for (int j = threadIdx.x; j < p.L; j += 256) out[p.cnt + j] = (int32_t)loc[j];
   }
-  if (threadIdx.x == 0 && p.counts) p.counts[row] = p.cnt + (p.local ? p.L : 0);
+  const int total = p.cnt + (p.local ? p.L : 0);
+  for (int j = total + threadIdx.x; j < p.zero_to; j += 256) out[j] = 0;   // the rest of the row: defined (zero)
+  if (threadIdx.x == 0 && p.counts) p.counts[row] = total;
 }
 
 int launch_remap_concat_lists(const RemapListParams& p, hipStream_t stream) {

@@ -455,11 +455,11 @@ def topk_token_lists(scores, k: int, out_len: Optional[int] = None, order: str =
     _require(0 <= k <= Lk, lambda: f"k = {k} must lie in [0, Lk = {Lk}]")
     out_len = Lk if out_len is None else int(out_len)
     _require(out_len >= k, "out_len must be at least k")
-    idx = torch.zeros(sc.shape[:-1] + (out_len,), dtype=torch.int32, device=sc.device)
+    idx = torch.empty(sc.shape[:-1] + (out_len,), dtype=torch.int32, device=sc.device)   # the kernel zeroes the tail
     cnt = torch.empty(sc.shape[:-1], dtype=torch.int32, device=sc.device)
     with _on_device(sc):
         st = _lib.load().lvar_topk_token_lists(sc.data_ptr(), Lk, idx.data_ptr(), out_len, cnt.data_ptr(),
-                                              rows, Lk, k, _stream(sc))
+                                              rows, Lk, k, out_len, _stream(sc))
     _lib.check(st, "lvar_topk_token_lists")
     if order == "value" and k > 0:
         sel = idx[..., :k].long()
@@ -494,11 +494,11 @@ def remap_concat_lists(src_indices, src_count: int, cur_q_len: int, cur_k_len: i
         L = loc.shape[1]
     out_len = int(cur_k_len) if out_len is None else int(out_len)
     _require(cnt + L <= out_len, lambda: f"list length {cnt + L} exceeds the output width {out_len}")
-    out = torch.zeros((B, H, Gk, out_len), dtype=torch.int32, device=src.device)
+    out = torch.empty((B, H, Gk, out_len), dtype=torch.int32, device=src.device)    # the kernel zeroes the tail
     counts = torch.empty((B, H, Gk), dtype=torch.int32, device=src.device)
     with _on_device(src):
         st = _lib.load().lvar_remap_concat_lists(src.data_ptr(), Ks, Ks, _ptr(loc), L, L, out.data_ptr(), out_len,
-                                                counts.data_ptr(), B * H, Gs, Gk, cnt, int(cur_k_len), _stream(src))
+                                                counts.data_ptr(), B * H, Gs, Gk, cnt, int(cur_k_len), out_len, _stream(src))
     _lib.check(st, "lvar_remap_concat_lists")
     return out, counts
 

@@ -71,14 +71,15 @@ def test_list_build_and_upsample_argument_validation(lib):
     null = LvarTensor(None, 0, 0, 0)
     fake = LvarTensor(0x1000, 128 * 16 * 128, 16 * 128, 128)
     one = ctypes.c_void_p(0x2000)
-    assert lib.lvar_topk_token_lists(None, 100, one, 100, one, 4, 100, 10, None) == -1            # no scores
-    assert lib.lvar_topk_token_lists(one, 100, one, 100, one, 4, 100, 101, None) == -1            # k > Lk
-    assert lib.lvar_topk_token_lists(one, 99, one, 100, one, 4, 100, 10, None) == -1              # row stride < Lk
-    assert lib.lvar_topk_token_lists(one, 100, one, 5, one, 4, 100, 10, None) == -1               # output row shorter than k
-    assert lib.lvar_topk_token_lists(one, 100, one, 100, one, 0, 100, 10, None) == 0              # no rows: nothing to launch
-    assert lib.lvar_remap_concat_lists(one, 100, 100, None, 0, 8, one, 200, one, 2, 3, 4, 64, 500, None) == -1   # local run without a table
-    assert lib.lvar_remap_concat_lists(one, 100, 100, one, 8, 8, one, 70, one, 2, 3, 4, 64, 500, None) == -1     # 64 + 8 > output row
-    assert lib.lvar_remap_concat_lists(one, 100, 100, None, 0, 0, one, 64, one, 2, 0, 4, 64, 500, None) == -1    # no source groups
+    assert lib.lvar_topk_token_lists(None, 100, one, 100, one, 4, 100, 10, 0, None) == -1            # no scores
+    assert lib.lvar_topk_token_lists(one, 100, one, 100, one, 4, 100, 101, 0, None) == -1            # k > Lk
+    assert lib.lvar_topk_token_lists(one, 99, one, 100, one, 4, 100, 10, 0, None) == -1              # row stride < Lk
+    assert lib.lvar_topk_token_lists(one, 100, one, 5, one, 4, 100, 10, 0, None) == -1               # output row shorter than k
+    assert lib.lvar_topk_token_lists(one, 100, one, 100, one, 4, 100, 10, 101, None) == -1           # zero fill beyond the row
+    assert lib.lvar_topk_token_lists(one, 100, one, 100, one, 0, 100, 10, 0, None) == 0              # no rows: nothing to launch
+    assert lib.lvar_remap_concat_lists(one, 100, 100, None, 0, 8, one, 200, one, 2, 3, 4, 64, 500, 0, None) == -1   # local run without a table
+    assert lib.lvar_remap_concat_lists(one, 100, 100, one, 8, 8, one, 70, one, 2, 3, 4, 64, 500, 0, None) == -1     # 64 + 8 > output row
+    assert lib.lvar_remap_concat_lists(one, 100, 100, None, 0, 0, one, 64, one, 2, 0, 4, 64, 500, 0, None) == -1    # no source groups
     assert lib.lvar_mask_to_lists(one, 10, one, 10, one, 3, 10, 0, None) == -1                    # multiple_of must be positive
     assert lib.lvar_mask_to_lists(one, 10, one, 9, one, 3, 10, 1, None) == -1                     # output row shorter than n
     assert lib.lvar_mask_to_lists(one, 10, one, 10, one, 0, 10, 1, None) == 0

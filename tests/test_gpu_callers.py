@@ -366,3 +366,9 @@ def test_compiled_dense_binding_matches_ctypes_path():
     assert torch.equal(o3, o_ref)
     with pytest.raises((TypeError, ValueError)):
         ops.dense_attn(qg.half(), kg.half(), vg.half())
+    # a scale that is not a Python float (numpy scalar, 0-dim tensor) takes the same path with the same bits
+    import numpy as np
+    o_f, (M_f, _) = ops.dense_attn(qg, kg, vg, 0.07)
+    for sc in (np.float32(0.07), torch.tensor(0.07), torch.tensor(0.07, device="cuda"), np.float64(0.07)):
+        o_s, (M_s, _) = ops.dense_attn(qg, kg, vg, sc)
+        assert (o_s.float() - o_f.float()).abs().max().item() < 1e-2 and (M_s - M_f).abs().max().item() < 1e-3
