@@ -65,7 +65,7 @@ typedef struct {
 int64_t lvar_attn_workspace_bytes(int head_dim);
 
 /* Workgroups a *_ws_fwd launch of these sizes would run as a balanced launch on the current device, 0 if it
- * would run as the plain launch; kind 0 = dense, 1 = block list (block_k 64 or 128, list_len = nk_max),
+ * would run as the plain launch; kind 0 = dense, 1 = block list (group_rows = block_q, block_k 64, 128 or 256, list_len = nk_max; 64-row query blocks always run as the plain launch),
  * 2 = token list (group_rows, list_len = idx_row_stride).  Pure planning: nothing is launched. */
 int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, int H, int Lq, int Lk, int list_len,
                                   int head_dim, lvar_workspace_t workspace);
@@ -192,7 +192,9 @@ int lvar_csp_attn_upsample_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_
  * kv_num_blocks int32 [B,H,nQ] (stride_nb_b, stride_nb_h, 1), kv_indices int32
  * [B,H,nQ,nk_max] (stride_ki_b, stride_ki_h, stride_ki_q, 1); a stride of 0 broadcasts.
  * kv_num_blocks entries are clamped to [0, nk_max].
- * block_q in {128}, block_k in {64, 128}; edge blocks are clipped to Lq / Lk.
+ * block_q = 64 or a multiple of 128, block_k in {64, 128, 256}; edge blocks are clipped to Lq / Lk.  Query blocks of
+ * 128 rows are the fast shape (one 4-wave workgroup per block); 64-row blocks run as 2-wave workgroups (the 64 x 64
+ * blocks of the reference's small configurations), larger ones as several 128-row workgroups that share a list.
  * A query block with no key block yields o = 0, M = -inf, L = 1.
  */
 int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o,
@@ -221,7 +223,7 @@ int lvar_block_sparse_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_
  * counterpart in the reference; it is for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments, results and balanced-launch
  * rule as lvar_block_sparse_attn_ws_fwd given a zeroed workspace of LVAR_STATIC_SCRATCH_BYTES.
- * Limits: B * H * ceil(Lq / 128) <= LVAR_STATIC_MAX_QUERY_TILES and head_dim <= 128, else LVAR_ETOOBIG (larger
+ * Limits: B * H * ceil(Lq / 128) (ceil(Lq / 64) for 64-row query blocks) <= LVAR_STATIC_MAX_QUERY_TILES and head_dim <= 128, else LVAR_ETOOBIG (larger
  * launches have enough query tiles to fill the chip: use lvar_block_sparse_attn_fwd).  All calls on one GPU share
  * that GPU's buffer: calls that overlap in time on one GPU (different streams or threads) race.
  */

@@ -207,8 +207,8 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       // offset (row within the first instruction, swizzled chunk: the swizzle does not depend on the
       // slot) is a constant and tile and slot only move a scalar offset.
       const int row0 = __builtin_amdgcn_readfirstlane(rows[0]);  // wave-uniform for block lists
-      if (MODE == MODE_BLOCK && row0 >= 0 && row0 <= p.Lk - 64) {   // anything else takes the clamped path below
-        static_assert(MODE != MODE_BLOCK || (FW * RPI) % 16 == 0, "slots of one wave must be a swizzle period (16 rows) apart");
+      // (needs the slots of one wave a swizzle period, 16 rows, apart: not so for two waves at head_dim 128)
+      if (MODE == MODE_BLOCK && (FW * RPI) % 16 == 0 && row0 >= 0 && row0 <= p.Lk - 64) {   // anything else takes the clamped path below
         const int trow0 = fwave * RPI + lrow;
         const int voff = trow0 * srb + ((lcs ^ (is_v ? Swz<D>::fv(trow0) : Swz<D>::fk(trow0))) << 4);
 #pragma unroll
@@ -907,7 +907,8 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
     const bool dense = (MODE == MODE_BLOCK && p.list == nullptr);
     const int64_t per_tile = (MODE == MODE_BLOCK) ? (p.list ? p.list_len : (p.Lk + 63) / 64) : (p.list_len + 63) / 64;
     const int sub = (MODE == MODE_BLOCK && p.list) ? p.sub_shift : 0;
-    p.sk_wgs = p.sk_ws ? sk_plan(p.total_wg, NWAVES, sk_slot_floats(D, MODE, NWAVES), per_tile, sub, p.sk_ws_bytes,
+    // (64-row query blocks always take the plain launch)
+    p.sk_wgs = (p.sk_ws && NWAVES != 2) ? sk_plan(p.total_wg, NWAVES, sk_slot_floats(D, MODE, NWAVES), per_tile, sub, p.sk_ws_bytes,
                                  p.sk_min_share, p.sk_min_piece) : 0;
     p.sk_uniform_n = 0;
     if (p.sk_wgs > 0 && dense) {
@@ -917,7 +918,7 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
       const int n = sk_worth_cutting(U, S, p.total_wg, p.sk_wgs) ? sk_pieces(T, S, p.sk_min_piece) : 1;
       if (n > 1 && (int64_t)n * p.total_wg <= 2 * p.sk_wgs) p.sk_uniform_n = n; else p.sk_wgs = 0;   // whole tiles: the plain launch
     }
-    if (p.sk_wgs > 0) {
+    if constexpr (NWAVES != 2) if (p.sk_wgs > 0) {
       p.sk_counters = (int*)p.sk_ws;
       p.sk_slots = (float*)((char*)p.sk_ws + SK_COUNTER_BYTES + sk_plan_bytes(p.sk_wgs));
       int grid_sk;
@@ -951,6 +952,8 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
 template <int D>
 static int launch_d(const AttnParams& p, int mode, bool accum, bool lse_only, int nwaves, hipStream_t s) {
   if (mode == MODE_BLOCK) {
+    if (nwaves == 2 && !lse_only) return launch_one<D, 2, MODE_BLOCK, false, false>(p, s);   // 64-row query blocks
+    if (nwaves != 4) return LVAR_EUNSUPPORTED;
     return lse_only ? launch_one<D, 4, MODE_BLOCK, false, true>(p, s) : launch_one<D, 4, MODE_BLOCK, false, false>(p, s);
   } else if (mode == MODE_GATHER) {
     if (nwaves == 8) return launch_one<D, 8, MODE_GATHER, true, false>(p, s);

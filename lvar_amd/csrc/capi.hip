@@ -230,7 +230,8 @@ static int block_sparse_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
   if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
   if (!kv_num_blocks || !kv_indices || nk_max <= 0 || o.stride_row <= 0) return LVAR_EINVAL;
-  if (block_q != 128 || (block_k != 64 && block_k != 128)) return LVAR_EUNSUPPORTED;
+  // query blocks of 64 rows (two-wave workgroups) or a multiple of 128 rows (128-row workgroups that share a list)
+  if ((block_q != 64 && (block_q <= 0 || block_q % 128 != 0)) || (block_k != 64 && block_k != 128 && block_k != 256)) return LVAR_EUNSUPPORTED;
   AttnParams p{};
   fill_qkv(p, q, k, v);
   p.o = (bf16_t*)o.ptr; p.o_sb = o.stride_b; p.o_sh = o.stride_h; p.o_sr = o.stride_row;
@@ -242,9 +243,9 @@ static int block_sparse_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v
   p.cnt_sb = stride_nb_b; p.cnt_sh = stride_nb_h;
   p.list_len = nk_max;
   p.group_rows = block_q;
-  p.sub_shift = (block_k == 128) ? 1 : 0;
+  p.sub_shift = (block_k == 256) ? 2 : (block_k == 128) ? 1 : 0;
   if (!attach_workspace(p, ws)) return LVAR_EINVAL;
-  return launch_attn(p, head_dim, MODE_BLOCK, false, false, 4, (hipStream_t)stream);
+  return launch_attn(p, head_dim, MODE_BLOCK, false, false, block_q == 64 ? 2 : 4, (hipStream_t)stream);
 }
 
 int lvar_block_sparse_attn_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
@@ -272,8 +273,10 @@ int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, 
   int nwaves = 4, mode = MODE_BLOCK, sub = 0;
   int64_t per_tile = (Lk + 63) / 64;
   if (kind == 1) {
-    if (block_k != 64 && block_k != 128) return LVAR_EUNSUPPORTED;
-    sub = block_k == 128 ? 1 : 0;
+    if (block_k != 64 && block_k != 128 && block_k != 256) return LVAR_EUNSUPPORTED;
+    if (group_rows == 64) return 0;   // 64-row query blocks always take the plain launch
+    if (group_rows <= 0 || group_rows % 128 != 0) return LVAR_EUNSUPPORTED;
+    sub = block_k == 256 ? 2 : block_k == 128 ? 1 : 0;
     per_tile = list_len;
   } else if (kind == 2) {
     nwaves = gather_waves(group_rows);
@@ -295,7 +298,8 @@ int lvar_block_sparse_attn_static_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_ten
                                       int head_dim, float scale, void* stream) {
   if (B <= 0 || H <= 0 || Lq <= 0) return LVAR_EINVAL;
   // the scratch holds the counters and the item table of at most LVAR_STATIC_MAX_QUERY_TILES query tiles
-  const int64_t tiles = (int64_t)B * H * ((Lq + 127) / 128);
+  const int wg_rows = block_q == 64 ? 64 : 128;
+  const int64_t tiles = (int64_t)B * H * ((Lq + wg_rows - 1) / wg_rows);
   if (tiles > LVAR_STATIC_MAX_QUERY_TILES || head_dim > 128) return LVAR_ETOOBIG;
   void* ptr = static_scratch();
   if (!ptr) return LVAR_ELAUNCH;

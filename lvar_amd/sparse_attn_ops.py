@@ -384,7 +384,8 @@ def block_sparse_attn(q, k, v, kv_num_blocks, kv_indices, block_q: int = 128, bl
     _check_qkv(q, k, v)
     B, H, Lq, d = q.shape
     Lk = k.shape[2]
-    _require(block_q == 128 and block_k in (64, 128), "block shape must be (128,64) or (128,128)")
+    _require((block_q == 64 or (block_q > 0 and block_q % 128 == 0)) and block_k in (64, 128, 256),
+             "block_q must be 64 or a multiple of 128, block_k 64, 128 or 256")
     nQ = (Lq + block_q - 1) // block_q
     _require(kv_num_blocks.dim() == 3 and kv_indices.dim() == 4, "kv_num_blocks must be [B,H,nQ], kv_indices [B,H,nQ,nKmax]")
     _require(kv_num_blocks.shape[2] == nQ and kv_indices.shape[2] == nQ,

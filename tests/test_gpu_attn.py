@@ -246,6 +246,60 @@ def test_block_sparse_attn(B, H, Lq, Lk, d, bk, density):
     check_lse(M, L, M_ref, L_ref)
 
 
+@pytest.mark.parametrize("B,H,Lq,Lk,d,bq,bk,density", [
+    (2, 3, 256, 680, 64, 64, 64, 0.5),     # the 64 x 64 blocks of the VAR-d16 benchmark case; last key block 40 keys
+    (1, 2, 200, 300, 128, 64, 64, 0.4),    # two-wave workgroups at head_dim 128, ragged Lq (200 = 3 * 64 + 8)
+    (1, 2, 150, 700, 128, 64, 128, 0.5),   # 64-row query blocks against 128-key blocks
+    (1, 2, 600, 1000, 128, 256, 64, 0.3),  # 256-row query blocks: two workgroups share a list; last block 88 rows
+    (1, 2, 384, 1100, 64, 384, 256, 0.6),  # 256-key blocks (four tiles per entry); last one has 76 keys
+    (1, 1, 128, 900, 128, 128, 256, 1.0),  # every 256-key block; the last block's tail tiles are empty
+])
+def test_block_sparse_attn_block_shapes(B, H, Lq, Lk, d, bq, bk, density):
+    """Block shapes other than 128 x {64, 128}: 64-row query blocks, query blocks that span several workgroups,
+    256-key blocks; each against the oracle on a random list."""
+    from lvar_amd import sparse_attn_ops as ops
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=Lq + Lk + bq + bk)
+    nQ, nK = (Lq + bq - 1) // bq, (Lk + bk - 1) // bk
+    mask = _random_block_lists(B, H, nQ, nK, density, seed=Lk + bq)
+    num, idx = oracle.block_mask_to_lists(mask)
+    o_ref, M_ref, L_ref = oracle.block_sparse_attn(q, k, v, num, idx, bq, bk)
+    o, (M, L) = ops.block_sparse_attn(*dev(q, k, v), num.cuda(), idx.cuda(), bq, bk)
+    check_o(o, o_ref, f"block sparse {bq}x{bk}")
+    check_lse(M, L, M_ref, L_ref)
+
+
+def test_var_d16_pipeline_64x64_blocks():
+    """The CPU-runnable benchmark case end to end on the GPU (B2 H16 d64 Lq256 Lk680, N(0,1) inputs, scale 1/8):
+    dense attention -> colsum over all 256 queries -> per-64-key block sums -> top 50 % = 5 of 11 key blocks per
+    (batch, head) -> block-sparse attention with 64 x 64 blocks; every stage against the oracle, the block
+    selection bit-exact on the same block sums."""
+    from lvar_amd import mask_build as mb
+    from lvar_amd import sparse_attn_ops as ops
+    B, H, Lq, Lk, d = 2, 16, 256, 680, 64
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=2024)
+    qg, kg, vg = dev(q, k, v)
+    o_ref, cs_ref, (M_ref, L_ref) = oracle.dense_colsum_attn(q, k, v, q_group_size=256)
+    o, (M, L) = ops.dense_attn(qg, kg, vg)
+    cs, bs = ops.colsum(qg, kg, q_group_size=256, lse=(M, L), return_block_sums=True)
+    check_o(o, o_ref, "dense")
+    check_lse(M, L, M_ref, L_ref)
+    assert cs.shape == (B, H, 1, Lk) and bs.shape == (B, H, 1, 11)
+    assert ((cs.cpu() - cs_ref).abs() <= 1e-3 * cs_ref.abs() + 1e-6).all()
+    assert ((bs.cpu() - oracle.key_block_sums(cs_ref, 64)).abs() <= 1e-3 * oracle.key_block_sums(cs_ref, 64)).all()
+    # selection on the GPU block sums, GPU list build against torch.topk on the same values
+    keep = oracle.indices_count(0.5, Lk, 64) // 64
+    assert keep == 5
+    nQ = Lq // 64
+    scores = bs.expand(B, H, nQ, 11).contiguous()
+    num, idx = ops.block_topk_lists(scores, keep)
+    top = torch.topk(bs.cpu()[:, :, 0], k=keep, dim=-1).indices.sort(-1).values.to(torch.int32)
+    assert bool((num == keep).all()) and torch.equal(idx.cpu()[..., :keep], top[:, :, None, :].expand(B, H, nQ, keep))
+    o_bs_ref, M2_ref, L2_ref = oracle.block_sparse_attn(q, k, v, num.cpu(), idx.cpu(), 64, 64)
+    o_bs, (M2, L2) = ops.block_sparse_attn(qg, kg, vg, num, idx, 64, 64)
+    check_o(o_bs, o_bs_ref, "block sparse 64x64")
+    check_lse(M2, L2, M2_ref, L2_ref)
+
+
 def test_block_sparse_full_mask_equals_dense_and_broadcast():
     from lvar_amd import sparse_attn_ops as ops
     B, H, Lq, Lk, d = 2, 3, 256, 777, 128
