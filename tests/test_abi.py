@@ -60,7 +60,8 @@ def test_argument_validation_without_device(lib):
     assert lib.lvar_csp_attn_fwd(fake, fake, fake, null, fake, None, None, one, one, 1, 16, 0, 1, 1, 16, 16, 128, 1.0, 1.0, None) == -1
     assert lib.lvar_dense_attn_rcp_fwd(fake, fake, fake, fake, None, 1, 1, 1, 16, 16, 128, 1.0, None) == -1                # no place for the row constant
     assert lib.lvar_csp_attn_fwd(fake, fake, fake, null, fake, None, None, None, one, 1, 16, 192, 1, 1, 16, 16, 128, 1.0, 1.0, None) == -1
-    assert lib.lvar_block_sparse_attn_fwd(fake, fake, fake, fake, None, None, one, 0, 0, one, 0, 0, 4, 4, 64, 64, 1, 1, 16, 16, 128, 1.0, None) == -2
+    assert lib.lvar_block_sparse_attn_fwd(fake, fake, fake, fake, None, None, one, 0, 0, one, 0, 0, 4, 4, 96, 64, 1, 1, 16, 16, 128, 1.0, None) == -2    # 96-row query blocks
+    assert lib.lvar_block_sparse_attn_fwd(fake, fake, fake, fake, None, None, one, 0, 0, one, 0, 0, 4, 4, 128, 32, 1, 1, 16, 16, 128, 1.0, None) == -2   # 32-key blocks
     wide = LvarTensor(0x1000, 1 << 30, 1 << 26, 1 << 23)                # row stride of 2^23 elements: beyond the 24-bit gather addressing
     assert lib.lvar_csp_attn_fwd(fake, wide, fake, null, fake, None, None, one, one, 1, 16, 192, 1, 1, 16, 16, 128, 1.0, 1.0, None) == -2
     assert lib.lvar_block_sparse_attn_fwd(fake, fake, fake, fake, None, None, None, 0, 0, one, 0, 0, 4, 4, 128, 64, 1, 1, 16, 16, 128, 1.0, None) == -1
