@@ -110,6 +110,35 @@ def device_summary():
     return out
 
 
+def sustained_mfma_rate():
+    """bf16 MFMA TFLOP/s of a register-resident loop (``lvar_amd/csrc/mfma_probe.hip``: every wave cycles through 8 A and
+    8 B fragments it holds in registers, 8 waves per CU) on random N(0,1)*0.5 operand bits and on all-zero bits, timed
+    on this box after the same settle period as the workload.  The clock under a matrix load follows the switching
+    activity of the operands, so the random-operand figure is the rate a bf16 MFMA kernel on this box can approach;
+    the published peak assumes the maximum clock.  None when the probe library is not built."""
+    import ctypes
+    path = os.path.join(ROOT, "lvar_amd", "liblvar_bench_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.lvar_probe_mfma.restype = ctypes.c_int
+    lib.lvar_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    blocks, iters = 2 * torch.cuda.get_device_properties(0).multi_processor_count, 2048
+    dst = torch.empty(blocks * 256, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    flops = blocks * 4.0 * iters * 16 * 32768
+    out = {"kernel": "mfma_probe_kernel: %d workgroups x 4 waves x %d x 16 MFMA 32x32x16" % (blocks, iters)}
+    g = torch.Generator().manual_seed(5)
+    for name, src in (("random_operands_tflops", (torch.randn(16 * 256 * 8, generator=g) * 0.5).to(torch.bfloat16).cuda()),
+                      ("zero_operands_tflops", torch.zeros(16 * 256 * 8, dtype=torch.bfloat16, device="cuda"))):
+        def fn():
+            st = lib.lvar_probe_mfma(src.data_ptr(), dst.data_ptr(), blocks, iters, stream)
+            assert st == 0, st
+        ms, _ = time_launches(fn, 30, 5)
+        out[name] = round(flops / ms / 1e9, 1)
+    return out
+
+
 def settle_clocks(fn, ms):
     """Keep the GPU busy with the workload for ``ms`` milliseconds.  After an idle period the part
     needs ~20 ms of load before its clocks settle (the first ~100 launches of the headline kernel
@@ -536,6 +565,7 @@ def main():
                "colsum_given_lse_us": round(cs_ms * 1e3, 1), "lse_pass_us": round(lse_ms * 1e3, 1),
                "colsum_plus_mask_build_ms": round(build_ms, 4), "speedup_vs_dense": round(dense_ms / ms, 3)}
 
+    probe = None if args.no_aux else sustained_mfma_rate()
     traffic, traffic_src = measured_traffic(wl)
     dev_sum = device_summary()
     # CU count x 4096 flop per clock x maximum engine clock, as the device reports them at run time; `peak` and
@@ -553,7 +583,8 @@ def main():
                      "peak_runtime": peak_rt, "frac_runtime": (round(tflops / peak_rt, 4) if peak_rt else None),
                      "flops_per_launch": flops, "host_wall_ms_per_step": round(wall_ms, 5),
                      "single_launch": single, "cache_state": "warm: back-to-back launches on the same inputs, no L2 flush",
-                     "settle_ms": SETTLE_MS},
+                     "settle_ms": SETTLE_MS, "sustained_mfma": probe,
+                     "frac_of_sustained_random": (round(tflops / probe["random_operands_tflops"], 4) if probe else None)},
         "cpu_baseline": cpu,
         "device": torch.cuda.get_device_name(0), "device_summary": dev_sum,
     }

@@ -65,6 +65,22 @@ def build_library(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+PROBE_PATH = os.path.join(HERE, "liblvar_bench_probe.so")
+
+
+def build_bench_probe(verbose: bool = False) -> str:
+    """Compile ``csrc/mfma_probe.hip`` (the sustained-MFMA-rate probe that ``bench.py`` times beside the
+    attention kernels) into its own small shared library.  Always rebuilds."""
+    tmp = PROBE_PATH + ".tmp"
+    out = _run([_hipcc(), *HIPCC_FLAGS, "-shared", os.path.join(CSRC, "mfma_probe.hip"), "-o", tmp])
+    os.replace(tmp, PROBE_PATH)
+    if verbose:
+        if out.strip():
+            print(out)
+        print("built", PROBE_PATH)
+    return PROBE_PATH
+
+
 BINDING_NAME = "_lvar_torch"
 BINDING_PATH = os.path.join(HERE, BINDING_NAME + ".so")
 
@@ -100,4 +116,5 @@ def build_torch_binding(verbose: bool = False) -> str:
 if __name__ == "__main__":
     build_library(verbose=True)
     build_torch_binding(verbose=True)
+    build_bench_probe(verbose=True)
     sys.exit(0)
