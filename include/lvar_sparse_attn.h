@@ -65,7 +65,7 @@ typedef struct {
 int64_t lvar_attn_workspace_bytes(int head_dim);
 
 /* Workgroups a *_ws_fwd launch of these sizes would run as a balanced launch on the current device, 0 if it
- * would run as the plain launch; kind 0 = dense, 1 = block list (group_rows = block_q, block_k 64, 128 or 256, list_len = nk_max; 64-row query blocks always run as the plain launch),
+ * would run as the plain launch; kind 0 = dense, 1 = block list (block_k 64, 128 or 256, list_len = nk_max; group_rows is only looked at for the value 64: query blocks of 64 rows always run as the plain launch),
  * 2 = token list (group_rows, list_len = idx_row_stride).  Pure planning: nothing is launched. */
 int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, int H, int Lq, int Lk, int list_len,
                                   int head_dim, lvar_workspace_t workspace);

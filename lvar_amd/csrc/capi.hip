@@ -274,8 +274,7 @@ int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, 
   int64_t per_tile = (Lk + 63) / 64;
   if (kind == 1) {
     if (block_k != 64 && block_k != 128 && block_k != 256) return LVAR_EUNSUPPORTED;
-    if (group_rows == 64) return 0;   // 64-row query blocks always take the plain launch
-    if (group_rows <= 0 || group_rows % 128 != 0) return LVAR_EUNSUPPORTED;
+    if (group_rows == 64) return 0;   // 64-row query blocks always take the plain launch; any other value: 128-row workgroups
     sub = block_k == 256 ? 2 : block_k == 128 ? 1 : 0;
     per_tile = list_len;
   } else if (kind == 2) {

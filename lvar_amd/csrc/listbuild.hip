@@ -7,9 +7,10 @@
 
 namespace lvar {
 
-// Order-preserving map float -> uint32 (larger float <=> larger key); -0.0 sorts below +0.0.
+// Order-preserving map float -> uint32 (larger float <=> larger key); -0.0 and +0.0 get the same key (adding +0.0
+// turns -0.0 into +0.0 and changes nothing else), so that they tie as they do in a comparison of the values.
 __device__ __forceinline__ uint32_t sort_key(float x) {
-  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const uint32_t u = __builtin_bit_cast(uint32_t, x + 0.0f);
   return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
 }
 
@@ -21,9 +22,9 @@ __device__ __forceinline__ int lanes_below(unsigned long long bal, int lane) {
 // Exact top-k per row by radix select.  One 512-thread workgroup per row; wave w owns the w-th
 // contiguous eighth of the (padded) row and every thread keeps its KPT keys in registers (KPT = 0:
 // rows too long for that are re-read from L2 in every pass).
-//   3 histogram passes (11, 11 and 10 bits, most significant first; LDS atomics) narrow the k-th
-//   largest key down to its exact value T and the number `need` of keys equal to T that belong to
-//   the selection (ties go to the smaller column);
+//   up to 3 histogram passes (11 bits each, most significant first, starting below the bits that all
+//   keys of the row share; LDS atomics) narrow the k-th largest key down to its exact value T and the
+//   number `need` of keys equal to T that belong to the selection (ties go to the smaller column);
 //   a counting pass gives every wave its number of selected keys, the last pass writes the selected
 //   columns in ascending order (ballot compaction).
 // ---------------------------------------------------------------------------------------------
@@ -51,11 +52,25 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
   const int cpw = KPT ? KPT : ((n + NT - 1) / NT);
   const int col0 = wave * cpw * 64 + lane;
   uint32_t keys[KPT ? KPT : 1];
+  uint32_t kmax = 0u, kmin = 0xffffffffu;   // over the real columns of this thread
   if (KPT) {
+    // All KPT loads are issued back to back (a branch around each would make them KPT dependent round trips):
+    // buffer loads bounded to the row, so that columns beyond n read as zero instead of reaching past the row.
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)s, 0, n * 4, 0x00020000);
+    uint32_t raw[KPT ? KPT : 1];
+#pragma unroll
+    for (int c = 0; c < KPT; c++) raw[c] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, col0 * 4, c * 256, 0);
 #pragma unroll
     for (int c = 0; c < KPT; c++) {
+      const bool real = col0 + c * 64 < n;
+      keys[c] = real ? sort_key(__builtin_bit_cast(float, raw[c])) : 0u;
+      kmax = max(kmax, keys[c]);
+      kmin = min(kmin, real ? keys[c] : 0xffffffffu);
+    }
+  } else {
+    for (int c = 0; c < cpw; c++) {
       const int j = col0 + c * 64;
-      keys[c] = (j < n) ? sort_key(s[j]) : 0u;
+      if (j < n) { const uint32_t key = sort_key(s[j]); kmax = max(kmax, key); kmin = min(kmin, key); }
     }
   }
   // visit(f): f(chunk, column, key) for every chunk of this wave (all 64 lanes call it together)
@@ -71,11 +86,27 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
     }
   };
 
-  uint32_t prefix = 0, pmask = 0;
+  // Column sums of one row sit in a narrow range: with the digits taken from the top of the key nearly every key
+  // would fall into a handful of bins of the first pass and the LDS atomics of a wave would serialise on them.  The
+  // bits that the largest and the smallest key of the row have in common are therefore taken as known, and the
+  // digits start at the first bit in which keys differ: `top` low bits are left to resolve, 11 at a time.
 #pragma unroll
-  for (int pass = 0; pass < 3; pass++) {
-    const int shift = (pass == 0) ? 21 : (pass == 1) ? 10 : 0;
-    const int bits = (pass == 2) ? 10 : 11;
+  for (int d = 32; d > 0; d >>= 1) {
+    kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d, 64));
+    kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, 64));
+  }
+  if (lane == 0) { wgt[wave] = (int)kmax; weq[wave] = (int)kmin; }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < NW; w++) { kmax = max(kmax, (uint32_t)wgt[w]); kmin = min(kmin, (uint32_t)weq[w]); }
+  const int top = 32 - __builtin_clz((kmax ^ kmin) | 1u) + (((kmax ^ kmin) == 0u) ? -1 : 0);   // 0 when all keys are equal
+  uint32_t pmask = (top >= 32) ? 0u : ~((1u << top) - 1u);
+  uint32_t prefix = kmax & pmask;
+  if (top == 0) __syncthreads();   // no pass below to separate these reads of wgt / weq from their reuse
+  for (int hi = top; hi > 0;) {
+    const int shift = max(0, hi - 11);
+    const int bits = hi - shift;
+    hi = shift;
     const int nbins = 1 << bits;
     for (int t = tid; t < nbins; t += NT) hist[t] = 0;
     __syncthreads();
@@ -112,7 +143,7 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
     prefix |= (uint32_t)sel[0] << shift;
     pmask |= (uint32_t)(nbins - 1) << shift;
     want = sel[1];
-    __syncthreads();
+    // (the next write of `sel` lies behind three more barriers: no barrier needed after these reads)
   }
   const uint32_t T = prefix;  // key of the k-th largest element
   const int need = want;      // selected keys equal to T (the first `need` of them by column)
@@ -130,15 +161,37 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
     eq_before += weq[w];
   }
   int eq_left = max(0, need - eq_before);
-  visit([&](int j, uint32_t key) {
+  // The selected columns of a wave are collected in a 128-entry ring in LDS (the histogram is no longer needed: the
+  // barrier above lies between its last read and these writes) and leave in full 64-entry, 256-byte stores instead
+  // of one partial store per chunk.  LDS operations of one wave complete in order, so the ring needs no barrier.
+  int* ring = hist + wave * 128;
+  int head = 0, fill = 0;   // wave-uniform
+  // the column numbers are formed again from a copy of col0 that the compiler cannot relate to the ones used above:
+  // kept alive from the loads they would be spilled, and their reloads would wait for every store in flight
+  int c0 = col0;
+  asm volatile("" : "+v"(c0));
+  auto emit = [&](int j, uint32_t key) {
     const bool is_gt = j < n && key > T, is_eq = j < n && key == T;
     const unsigned long long beq = __builtin_amdgcn_ballot_w64(is_eq);
     const bool keep = is_gt || (is_eq && lanes_below(beq, lane) < eq_left);
     const unsigned long long bk = __builtin_amdgcn_ballot_w64(keep);
-    if (keep) out[pos + lanes_below(bk, lane)] = j;
-    pos += __builtin_popcountll(bk);
+    if (keep) ring[(head + fill + lanes_below(bk, lane)) & 127] = j;
+    fill += __builtin_popcountll(bk);
     eq_left = max(0, eq_left - __builtin_popcountll(beq));
-  });
+    if (fill >= 64) {
+      out[pos + lane] = ring[(head + lane) & 127];
+      head = (head + 64) & 127;
+      pos += 64;
+      fill -= 64;
+    }
+  };
+  if (KPT) {
+#pragma unroll
+    for (int c = 0; c < KPT; c++) emit(c0 + c * 64, keys[c]);
+  } else {
+    visit(emit);
+  }
+  if (lane < fill) out[pos + lane] = ring[(head + lane) & 127];
 }
 
 int launch_topk_token_lists(const TopkListParams& p, hipStream_t stream) {

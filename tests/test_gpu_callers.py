@@ -190,6 +190,22 @@ def test_topk_token_lists_matches_oracle_set():
         exp = oracle.topk_token_set(x, k)
         assert torch.equal(idx[..., :k].cpu(), exp), (shape, k)
         assert bool((idx[..., k:] == 0).all())
+    # Rows whose values share most of their leading bits (what column sums look like): the digits of the radix
+    # select start below the common prefix.  Values in one binade; in a range of a few ulps (ties on every level);
+    # a row of two values one ulp apart; all-negative and sign-straddling narrow rows; -0.0 against +0.0.
+    base = torch.full((8, 4121), 0.0181)
+    x = base.clone()
+    x[0] += torch.rand(4121, generator=g) * 1e-3
+    x[1] = 0.0181 + torch.randint(0, 5, (4121,), generator=g).float() * 2.0 ** -29
+    x[2, ::2] = torch.nextafter(torch.tensor(0.0181), torch.tensor(1.0))
+    x[3] = -(0.0181 + torch.rand(4121, generator=g) * 1e-3)
+    x[4] = (torch.rand(4121, generator=g) - 0.5) * 1e-6
+    x[5] = torch.where(torch.rand(4121, generator=g) < 0.5, torch.tensor(-0.0), torch.tensor(0.0))
+    x[6] = torch.softmax(torch.randn(192, 4121, generator=g), -1).sum(0)
+    x[7, 100] = 5.0                                                     # one outlier above a constant row
+    for k in (1, 832, 2060, 4121):
+        idx, cnt = ops.topk_token_lists(x.cuda(), k)
+        assert torch.equal(idx[..., :k].cpu(), oracle.topk_token_set(x, k)), k
     x = torch.rand(2, 2, 3, 500, generator=g)
     idx, _ = ops.topk_token_lists(x.cuda(), 64, order="value")
     assert torch.equal(idx[..., :64].cpu().long(), torch.topk(x, 64, dim=-1).indices)   # distinct values: same order
