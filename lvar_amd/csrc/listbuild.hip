@@ -29,13 +29,21 @@ __device__ __forceinline__ int lanes_below(unsigned long long bal, int lane) {
 //   columns in ascending order (ballot compaction).
 // ---------------------------------------------------------------------------------------------
 constexpr int TOPK_BINS = 2048;
+constexpr int TOPK_CAND = 256;   // keys of the first pass's bin that are resolved by direct comparison
+
+// Key of a real column: never 0, which is the key of the padding columns beyond the row.  (Only a NaN with every
+// bit set maps to 0; it is lifted to 1.)  Padding keys are then below every real key: they never compare greater than
+// or equal to the threshold, and a histogram counts them at the very bottom, below the k real keys that are wanted.
+__device__ __forceinline__ uint32_t real_key(float x) { return max(sort_key(x), 1u); }
 
 template <int KPT, int NT>
 __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kernel(const TopkListParams p) {
   constexpr int NW = NT / 64;
   __shared__ int hist[TOPK_BINS];
+  __shared__ uint32_t cand[TOPK_CAND];
   __shared__ int wsum[NW];
   __shared__ int sel[2];  // chosen bin, keys still wanted inside it
+  __shared__ int ncand;
   __shared__ int wgt[NW], weq[NW];
   const int row = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -63,25 +71,29 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
 #pragma unroll
     for (int c = 0; c < KPT; c++) {
       const bool real = col0 + c * 64 < n;
-      keys[c] = real ? sort_key(__builtin_bit_cast(float, raw[c])) : 0u;
+      keys[c] = real ? real_key(__builtin_bit_cast(float, raw[c])) : 0u;
       kmax = max(kmax, keys[c]);
       kmin = min(kmin, real ? keys[c] : 0xffffffffu);
     }
   } else {
     for (int c = 0; c < cpw; c++) {
       const int j = col0 + c * 64;
-      if (j < n) { const uint32_t key = sort_key(s[j]); kmax = max(kmax, key); kmin = min(kmin, key); }
+      if (j < n) { const uint32_t key = real_key(s[j]); kmax = max(kmax, key); kmin = min(kmin, key); }
     }
   }
-  // visit(f): f(chunk, column, key) for every chunk of this wave (all 64 lanes call it together)
+  // visit(f): f(column, key) for every chunk of this wave (all 64 lanes call it together); padding columns have key 0.
+  // The column numbers are formed from a copy of col0 that the compiler cannot relate to the ones of the loads:
+  // kept alive from there they would be spilled, and their reloads would wait for every store in flight.
+  int c0 = col0;
+  asm volatile("" : "+v"(c0));
   auto visit = [&](auto&& f) {
     if (KPT) {
 #pragma unroll
-      for (int c = 0; c < KPT; c++) f(col0 + c * 64, keys[c]);
+      for (int c = 0; c < KPT; c++) f(c0 + c * 64, keys[c]);
     } else {
       for (int c = 0; c < cpw; c++) {
-        const int j = col0 + c * 64;
-        f(j, (j < n) ? sort_key(s[j]) : 0u);
+        const int j = c0 + c * 64;
+        f(j, (j < n) ? real_key(s[j]) : 0u);
       }
     }
   };
@@ -96,6 +108,7 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
     kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, 64));
   }
   if (lane == 0) { wgt[wave] = (int)kmax; weq[wave] = (int)kmin; }
+  if (tid == 0) ncand = 0;
   __syncthreads();
 #pragma unroll
   for (int w = 0; w < NW; w++) { kmax = max(kmax, (uint32_t)wgt[w]); kmin = min(kmin, (uint32_t)weq[w]); }
@@ -103,6 +116,7 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
   uint32_t pmask = (top >= 32) ? 0u : ~((1u << top) - 1u);
   uint32_t prefix = kmax & pmask;
   if (top == 0) __syncthreads();   // no pass below to separate these reads of wgt / weq from their reuse
+  bool first = true;
   for (int hi = top; hi > 0;) {
     const int shift = max(0, hi - 11);
     const int bits = hi - shift;
@@ -111,7 +125,7 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
     for (int t = tid; t < nbins; t += NT) hist[t] = 0;
     __syncthreads();
     visit([&](int j, uint32_t key) {
-      if (j < n && (key & pmask) == prefix) atomicAdd(&hist[(key >> shift) & (nbins - 1)], 1);
+      if ((key & pmask) == prefix) atomicAdd(&hist[(key >> shift) & (nbins - 1)], 1);
     });
     __syncthreads();
     // thread t owns the bpt bins nbins-1 - t*bpt .. (descending); find the bin holding the want-th key from the top
@@ -144,14 +158,49 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
     pmask |= (uint32_t)(nbins - 1) << shift;
     want = sel[1];
     // (the next write of `sel` lies behind three more barriers: no barrier needed after these reads)
+    if (first && hi > 0) {
+      // After the first pass the chosen bin usually holds a few dozen keys.  They are copied to LDS, and if they
+      // fit, every one of them counts the candidates above it: the one with fewer than `want` above and at least
+      // `want` at or above is the threshold, and the other passes are not needed.
+      first = false;
+      visit([&](int j, uint32_t key) {
+        const bool m = (key & pmask) == prefix;
+        const unsigned long long bm = __builtin_amdgcn_ballot_w64(m);
+        if (bm != 0ull) {
+          int base = 0;
+          if (lane == 0) base = atomicAdd(&ncand, __builtin_popcountll(bm));
+          base = __builtin_amdgcn_readfirstlane(base);
+          const int at = base + lanes_below(bm, lane);
+          if (m && at < TOPK_CAND) cand[at] = key;
+        }
+      });
+      __syncthreads();
+      const int nc = ncand;
+      if (nc <= TOPK_CAND) {
+        if (tid < nc) {
+          const uint32_t kt = cand[tid];
+          int above = 0, at_or_above = 0;
+          for (int u = 0; u < nc; u++) {
+            const uint32_t ku = cand[u];
+            above += ku > kt;
+            at_or_above += ku >= kt;
+          }
+          if (above < want && want <= at_or_above) { sel[0] = (int)kt; sel[1] = want - above; }   // equal keys write equal values
+        }
+        __syncthreads();
+        prefix = (uint32_t)sel[0];
+        want = sel[1];
+        break;
+      }
+    }
   }
   const uint32_t T = prefix;  // key of the k-th largest element
   const int need = want;      // selected keys equal to T (the first `need` of them by column)
 
   int gt = 0, eq = 0;
   visit([&](int j, uint32_t key) {
-    gt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(j < n && key > T));
-    eq += __builtin_popcountll(__builtin_amdgcn_ballot_w64(j < n && key == T));
+    gt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(key > T));
+    eq += __builtin_popcountll(__builtin_amdgcn_ballot_w64(key == T));
   });
   if (lane == 0) { wgt[wave] = gt; weq[wave] = eq; }
   __syncthreads();
@@ -166,31 +215,22 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
   // of one partial store per chunk.  LDS operations of one wave complete in order, so the ring needs no barrier.
   int* ring = hist + wave * 128;
   int head = 0, fill = 0;   // wave-uniform
-  // the column numbers are formed again from a copy of col0 that the compiler cannot relate to the ones used above:
-  // kept alive from the loads they would be spilled, and their reloads would wait for every store in flight
-  int c0 = col0;
-  asm volatile("" : "+v"(c0));
-  auto emit = [&](int j, uint32_t key) {
-    const bool is_gt = j < n && key > T, is_eq = j < n && key == T;
-    const unsigned long long beq = __builtin_amdgcn_ballot_w64(is_eq);
-    const bool keep = is_gt || (is_eq && lanes_below(beq, lane) < eq_left);
-    const unsigned long long bk = __builtin_amdgcn_ballot_w64(keep);
-    if (keep) ring[(head + fill + lanes_below(bk, lane)) & 127] = j;
+  visit([&](int j, uint32_t key) {
+    unsigned long long bk = __builtin_amdgcn_ballot_w64(key > T);
+    const unsigned long long beq = __builtin_amdgcn_ballot_w64(key == T);
+    if (beq != 0ull && eq_left > 0) {   // keys equal to the threshold: the first eq_left of them by column
+      bk |= __builtin_amdgcn_ballot_w64(key == T && lanes_below(beq, lane) < eq_left);
+      eq_left = max(0, eq_left - __builtin_popcountll(beq));
+    }
+    if ((bk >> lane) & 1ull) ring[(head + fill + lanes_below(bk, lane)) & 127] = j;
     fill += __builtin_popcountll(bk);
-    eq_left = max(0, eq_left - __builtin_popcountll(beq));
     if (fill >= 64) {
       out[pos + lane] = ring[(head + lane) & 127];
       head = (head + 64) & 127;
       pos += 64;
       fill -= 64;
     }
-  };
-  if (KPT) {
-#pragma unroll
-    for (int c = 0; c < KPT; c++) emit(c0 + c * 64, keys[c]);
-  } else {
-    visit(emit);
-  }
+  });
   if (lane < fill) out[pos + lane] = ring[(head + lane) & 127];
 }
 
