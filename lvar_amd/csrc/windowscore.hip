@@ -7,7 +7,7 @@
 
 namespace lvar {
 
-constexpr int WS_KEYS = 256;   // keys per workgroup
+constexpr int WS_KEYS = 512;   // keys per workgroup (every workgroup sums the window queries for itself: the more keys, the less that weighs)
 constexpr int WS_MAXR = 16;    // largest pool radius (kernel_size <= 33)
 
 template <int D>
@@ -32,13 +32,29 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const WinScoreParams
   // Row group g (LPR lanes, 16 bytes each) adds up the window rows g, g + RPP, ...; the RPP partial
   // sums meet in LDS.
   const int g = tid / LPR, l = tid - g * LPR;
+  constexpr int UN = 8;   // rows in flight per lane: the loads of a batch are issued together, not one per round trip
   {
     float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int i = g; i < p.W; i += RPP) {
-      const int row = max(0, min(p.Lq - 1, (int)win[i] - (p.Lk - p.Lq)));
-      const u32x4 qv4 = *(const u32x4*)(qb + (int64_t)row * p.q_sr + l * 8);
+    for (int i0 = g; i0 < p.W; i0 += RPP * UN) {
+      int rows[UN];
 #pragma unroll
-      for (int e = 0; e < 4; e++) { a[2 * e] += bf16_lo(qv4[e]); a[2 * e + 1] += bf16_hi(qv4[e]); }
+      for (int u = 0; u < UN; u++) {
+        const int i = i0 + u * RPP;
+        rows[u] = (int)win[min(i, p.W - 1)];
+      }
+      u32x4 qv4[UN];
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int row = max(0, min(p.Lq - 1, rows[u] - (p.Lk - p.Lq)));
+        qv4[u] = *(const u32x4*)(qb + (int64_t)row * p.q_sr + l * 8);
+      }
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        if (i0 + u * RPP < p.W) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) { a[2 * e] += bf16_lo(qv4[u][e]); a[2 * e + 1] += bf16_hi(qv4[u][e]); }
+        }
+      }
     }
 #pragma unroll
     for (int e = 0; e < 8; e++) part[g][l * 8 + e] = a[e];
@@ -55,19 +71,25 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const WinScoreParams
 #pragma unroll
   for (int e = 0; e < 8; e++) qv[e] = qs[l * 8 + e];
   const float pad = p.maxpool ? -INFINITY : 0.f;
-  for (int j = g; j < span; j += RPP) {
-    const int n = n0 + j;
-    float dot = 0.f;
-    if (n >= 0 && n < p.Lk) {
-      const u32x4 kv = *(const u32x4*)(kb + (int64_t)n * p.k_sr + l * 8);
+  for (int j0 = g; j0 < span; j0 += RPP * UN) {
+    u32x4 kv[UN];
 #pragma unroll
-      for (int e = 0; e < 4; e++) dot += bf16_lo(kv[e]) * qv[2 * e] + bf16_hi(kv[e]) * qv[2 * e + 1];
+    for (int u = 0; u < UN; u++) {
+      const int n = max(0, min(p.Lk - 1, n0 + j0 + u * RPP));   // clamped: the load is unconditional, its use is not
+      kv[u] = *(const u32x4*)(kb + (int64_t)n * p.k_sr + l * 8);
     }
 #pragma unroll
-    for (int m = LPR >> 1; m > 0; m >>= 1) dot += __shfl_xor(dot, m, 64);
-    if (l == 0) {
-      sc[j] = (n >= 0 && n < p.Lk) ? dot * p.scale : pad;
-      wm[j] = 0;
+    for (int u = 0; u < UN; u++) {
+      const int j = j0 + u * RPP, n = n0 + j;
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; e++) dot += bf16_lo(kv[u][e]) * qv[2 * e] + bf16_hi(kv[u][e]) * qv[2 * e + 1];
+#pragma unroll
+      for (int m = LPR >> 1; m > 0; m >>= 1) dot += __shfl_xor(dot, m, 64);
+      if (l == 0 && j < span) {
+        sc[j] = (n >= 0 && n < p.Lk) ? dot * p.scale : pad;
+        wm[j] = 0;
+      }
     }
   }
   __syncthreads();
@@ -78,12 +100,14 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const WinScoreParams
     if (j >= 0 && j < span) { sc[j] = -INFINITY; wm[j] = 1; }
   }
   __syncthreads();
-  const int n = chunk * WS_KEYS + tid;
-  if (n < p.Lk) {
-    float acc = p.maxpool ? -INFINITY : 0.f;
-    for (int e = 0; e <= 2 * r; e++) acc = p.maxpool ? fmaxf(acc, sc[tid + e]) : acc + sc[tid + e];
-    if (!p.maxpool) acc = acc / (float)p.ksize;
-    p.out[(int64_t)bh * p.Lk + n] = wm[tid + r] ? -INFINITY : acc;
+  for (int t = tid; t < WS_KEYS; t += 256) {
+    const int n = chunk * WS_KEYS + t;
+    if (n < p.Lk) {
+      float acc = p.maxpool ? -INFINITY : 0.f;
+      for (int e = 0; e <= 2 * r; e++) acc = p.maxpool ? fmaxf(acc, sc[t + e]) : acc + sc[t + e];
+      if (!p.maxpool) acc = acc / (float)p.ksize;
+      p.out[(int64_t)bh * p.Lk + n] = wm[t + r] ? -INFINITY : acc;
+    }
   }
 }
 
