@@ -202,56 +202,52 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
     // Issue the global->LDS loads of one tile (K or V) into the LDS buffer at byte address `dst`.
     // Written as inline assembly so that the compiler does not serialise later LDS reads of the
     // OTHER buffers behind these fills; completion is awaited with vmcnt(0) before the barrier.
-    auto issue = [&](const i32x4& rsrc, int srb, bool is_v, const int (&rows)[NR], uint32_t dst) {
+    // issue_slot: the s-th of the SLOTS fill instructions this wave contributes to a tile; issue: all of them.
+    auto issue_slot = [&](const i32x4& rsrc, int srb, bool is_v, const int (&rows)[NR], uint32_t dst, int s) {
+      const int i = fwave + s * FW;
+      if (!((NI % FW == 0) || i < NI)) return;
+      const uint32_t m0v = dst + i * 1024;
       // Block lists, tile fully inside K/V: the rows of a tile are consecutive, so the per-lane byte
       // offset (row within the first instruction, swizzled chunk: the swizzle does not depend on the
       // slot) is a constant and tile and slot only move a scalar offset.
-      const int row0 = __builtin_amdgcn_readfirstlane(rows[0]);  // wave-uniform for block lists
-      // (needs the slots of one wave a swizzle period, 16 rows, apart: not so for two waves at head_dim 128)
-      if (MODE == MODE_BLOCK && (FW * RPI) % 16 == 0 && row0 >= 0 && row0 <= p.Lk - 64) {   // anything else takes the clamped path below
+      // The buffer descriptor ends with the last key row, so the rows of a ragged last tile that lie beyond it read
+      // as zeros (they are masked in the softmax); the first row is never negative (finish_rows clamps the block).
+      // (Needs the slots of one wave a swizzle period, 16 rows, apart: not so for two waves at head_dim 128.)
+      if constexpr (MODE == MODE_BLOCK && (FW * RPI) % 16 == 0) {
+        const int row0 = __builtin_amdgcn_readfirstlane(rows[0]);  // wave-uniform for block lists
         const int trow0 = fwave * RPI + lrow;
         const int voff = trow0 * srb + ((lcs ^ (is_v ? Swz<D>::fv(trow0) : Swz<D>::fk(trow0))) << 4);
-#pragma unroll
-        for (int s = 0; s < SLOTS; s++) {
-          const int i = fwave + s * FW;
-          if ((NI % FW == 0) || i < NI) {
-            const int soff = (row0 + s * FW * RPI) * srb;
-            const uint32_t m0v = dst + i * 1024;
-            asm volatile(
-                "s_mov_b32 m0, %0\n\t"
-                "s_nop 0\n\t"
-                "buffer_load_dwordx4 %1, %2, %3 offen lds"
-                :
-                : "s"(m0v), "v"(voff), "s"(rsrc), "s"(soff)
-                : "memory");
-          }
-        }
+        const int soff = (row0 + s * FW * RPI) * srb;
+        asm volatile(
+            "s_mov_b32 m0, %0\n\t"
+            "s_nop 0\n\t"
+            "buffer_load_dwordx4 %1, %2, %3 offen lds"
+            :
+            : "s"(m0v), "v"(voff), "s"(rsrc), "s"(soff)
+            : "memory");
         return;
       }
-#pragma unroll
-      for (int s = 0; s < SLOTS; s++) {
-        const int i = fwave + s * FW;
-        if ((NI % FW == 0) || i < NI) {
-          const int trow = i * RPI + lrow;
-          const int chunk = lcs ^ (is_v ? Swz<D>::fv(trow) : Swz<D>::fk(trow));
-          int voff;
-          if (MODE == MODE_GATHER) {
-            // token rows and row strides are below 2^24 (checked on the host): one full-rate 24-bit multiply-add
-            voff = (int)(((unsigned)rows[s < NR ? s : 0] & 0xffffffu) * ((unsigned)srb & 0xffffffu) + (unsigned)(chunk * 16));
-          } else {
-            const int grow = max(0, min(rows[0] + trow, p.Lk - 1));
-            voff = grow * srb + chunk * 16;
-          }
-          const uint32_t m0v = dst + i * 1024;
-          asm volatile(
-              "s_mov_b32 m0, %0\n\t"
-              "s_nop 0\n\t"
-              "buffer_load_dwordx4 %1, %2, 0 offen lds"
-              :
-              : "s"(m0v), "v"(voff), "s"(rsrc)
-              : "memory");  // m0 is scratch here: nothing else in this kernel keeps a value in it
-        }
+      const int trow = i * RPI + lrow;
+      const int chunk = lcs ^ (is_v ? Swz<D>::fv(trow) : Swz<D>::fk(trow));
+      int voff;
+      if (MODE == MODE_GATHER) {
+        // token rows and row strides are below 2^24 (checked on the host): one full-rate 24-bit multiply-add
+        voff = (int)(((unsigned)rows[s < NR ? s : 0] & 0xffffffu) * ((unsigned)srb & 0xffffffu) + (unsigned)(chunk * 16));
+      } else {
+        const int grow = max(0, min(rows[0] + trow, p.Lk - 1));
+        voff = grow * srb + chunk * 16;
       }
+      asm volatile(
+          "s_mov_b32 m0, %0\n\t"
+          "s_nop 0\n\t"
+          "buffer_load_dwordx4 %1, %2, 0 offen lds"
+          :
+          : "s"(m0v), "v"(voff), "s"(rsrc)
+          : "memory");  // m0 is scratch here: nothing else in this kernel keeps a value in it
+    };
+    auto issue = [&](const i32x4& rsrc, int srb, bool is_v, const int (&rows)[NR], uint32_t dst) {
+#pragma unroll
+      for (int s = 0; s < SLOTS; s++) issue_slot(rsrc, srb, is_v, rows, dst, s);
     };
 
     // valid keys of tile t of a token list (only the last tile can be ragged)
@@ -435,11 +431,30 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
     auto body = [&](int t, auto par, auto masked, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1) {
       constexpr int PAR = decltype(par)::value;
       constexpr bool MASKED = decltype(masked)::value;
+      // The fills of V(t+1) and K(t+2) are not issued in one burst up front (a wave spends tens of cycles on each and
+      // the matrix cores would sit idle meanwhile) but one by one between the QK MFMAs, where their issue runs in the
+      // shadow of the MFMA before.  NFILL instructions, one every FSTRIDE steps; if there are more than steps, up front.
+      constexpr int NQK_ = 2 * KS;
+      constexpr int NFILL = NPROD ? 0 : (LSE_ONLY ? SLOTS : 2 * SLOTS);
+      constexpr int FSTRIDE = (MODE == MODE_BLOCK && (FW * RPI) % 16 == 0 && NFILL > 0 && NFILL <= NQK_) ? NQK_ / NFILL : 0;
+      const bool fill_k = t + 2 < T;
+      auto fill_step = [&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        if constexpr (FSTRIDE > 0) {
+          if constexpr (j % FSTRIDE == 0 && j / FSTRIDE < NFILL) {
+            constexpr int f = j / FSTRIDE;
+            if constexpr (!LSE_ONLY && f < SLOTS) issue_slot(vrsrc, v_srb, true, rows_v, lds0 + (3 - PAR) * TILE, f);
+            else if (fill_k) issue_slot(krsrc, k_srb, false, rows_k, lds0 + PAR * TILE, LSE_ONLY ? f : f - SLOTS);
+          }
+        }
+      };
       if (NPROD) {
         nv3 = nvalid_gather(t + 3);
       } else {
-        if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows_v, lds0 + (3 - PAR) * TILE);
-        if (t + 2 < T) issue(krsrc, k_srb, false, rows_k, lds0 + PAR * TILE);
+        if constexpr (FSTRIDE == 0) {
+          if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows_v, lds0 + (3 - PAR) * TILE);
+          if (fill_k) issue(krsrc, k_srb, false, rows_k, lds0 + PAR * TILE);
+        }
         if (t + 3 < T) finish_rows(t + 3, raw, rows_n, nv3);
         if (t + 4 < T) prefetch_raw(t + 4, raw);
       }
@@ -509,6 +524,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
         else if constexpr (j == 1) n1 = mfma32(frag[j], qf[0], f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0});
         else if constexpr (j & 1) n1 = mfma32(frag[j], qf[j >> 1], n1);
         else n0 = mfma32(frag[j], qf[j >> 1], n0);
+        fill_step(jc);
         softmax_step(jc);
         __builtin_amdgcn_sched_barrier(0);
       });
