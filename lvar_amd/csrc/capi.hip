@@ -42,9 +42,11 @@ bool view_ok(const lvar_tensor_t& t) {
   return t.ptr && aligned16(t.ptr) && t.stride_b % 8 == 0 && t.stride_h % 8 == 0 && t.stride_row % 8 == 0;
 }
 
-// K/V rows are addressed with 32-bit byte offsets inside one (batch, head) slice
+// K/V rows are addressed with 32-bit byte offsets inside one (batch, head) slice.  The fills of a ragged last tile
+// (or of the last tiles of a 256-key block) form offsets of up to 319 rows beyond the last key before the buffer
+// descriptor's bound turns them into zeros: those offsets must not wrap either.
 bool kv_span_ok(const lvar_tensor_t& t, int Lk, int head_dim) {
-  return t.stride_row > 0 && (double)t.stride_row * 2.0 * Lk + head_dim * 2.0 < 2147483647.0;
+  return t.stride_row > 0 && (double)t.stride_row * 2.0 * ((double)Lk + 320.0) + head_dim * 2.0 < 2147483647.0;
 }
 
 bool shape_ok(int B, int H, int Lq, int Lk, float scale) {
