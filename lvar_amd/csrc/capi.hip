@@ -45,8 +45,9 @@ bool view_ok(const lvar_tensor_t& t) {
 // K/V rows are addressed with 32-bit byte offsets inside one (batch, head) slice.  The fills of a ragged last tile
 // (or of the last tiles of a 256-key block) form offsets of up to 319 rows beyond the last key before the buffer
 // descriptor's bound turns them into zeros: those offsets must not wrap either.
-bool kv_span_ok(const lvar_tensor_t& t, int Lk, int head_dim) {
-  return t.stride_row > 0 && (double)t.stride_row * 2.0 * ((double)Lk + 320.0) + head_dim * 2.0 < 2147483647.0;
+// (Token lists clamp every gathered row to the last key: pad_rows = 0.)
+bool kv_span_ok(const lvar_tensor_t& t, int Lk, int head_dim, int pad_rows = 320) {
+  return t.stride_row > 0 && (double)t.stride_row * 2.0 * ((double)Lk + pad_rows) + head_dim * 2.0 < 2147483647.0;
 }
 
 bool shape_ok(int B, int H, int Lq, int Lk, float scale) {
@@ -141,7 +142,7 @@ int lvar_colsum_fwd(lvar_tensor_t q, lvar_tensor_t k, const float* lse2, float* 
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !lse2 || !cs) return LVAR_EINVAL;
   if (kv_heads <= 0 || H % kv_heads != 0) return LVAR_EINVAL;
   if (q_group_size <= 0 || q_group_size % 32 != 0) return LVAR_EINVAL;
-  if (!kv_span_ok(q, Lq, head_dim)) return LVAR_EINVAL;
+  if (!kv_span_ok(q, Lq, head_dim, 0)) return LVAR_EINVAL;
   ColsumParams p{};
   p.q = (const bf16_t*)q.ptr; p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sr = q.stride_row;
   p.k = (const bf16_t*)k.ptr; p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sr = k.stride_row;
@@ -159,7 +160,7 @@ static int csp_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_te
                       float o_scale, float scale, const lvar_workspace_t* ws, void* stream) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
   if (o.stride_row <= 0 || (o_accum.ptr && (!view_ok(o_accum) || o_accum.stride_row <= 0))) return LVAR_EINVAL;
-  if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
+  if (!kv_span_ok(k, Lk, head_dim, 0) || !kv_span_ok(v, Lk, head_dim, 0)) return LVAR_EINVAL;
   // gathered rows are addressed with a 24-bit multiply: token index and row stride in bytes below 2^24
   if (Lk > (1 << 24) || k.stride_row * 2 >= (1 << 24) || v.stride_row * 2 >= (1 << 24)) return LVAR_EUNSUPPORTED;
   if (!indices || !counts || G <= 0 || idx_row_stride <= 0) return LVAR_EINVAL;
