@@ -471,12 +471,14 @@ def topk_token_lists(scores, k: int, out_len: Optional[int] = None, order: str =
 
 
 def remap_concat_lists(src_indices, src_count: int, cur_q_len: int, cur_k_len: int, local_indices=None,
-                       bm: int = 192, indices_pad_to: int = 1, out_len: Optional[int] = None):
+                       bm: int = 192, indices_pad_to: int = 1, out_len: Optional[int] = None, zero_tail: bool = True):
     """One-launch sparse-step key list: the decision-scale lists ``src_indices`` int32 ``[B,H,Gs,Ks]``
     (first ``src_count`` columns valid) are mapped to the ``Gk = ceil(cur_q_len / bm)`` query groups of the
     current scale (nearest group centre, half-to-even), clamped to ``[0, cur_k_len)``, and followed by
     the rows of ``local_indices`` int64 ``[Gk, L]`` (optional).  Returns ``(indices int32 [B,H,Gk,out_len],
-    counts int32 [B,H,Gk])``; ``out_len`` defaults to ``cur_k_len``.  Equals
+    counts int32 [B,H,Gk])``; ``out_len`` defaults to ``cur_k_len``.  The columns behind the list are zero unless
+    ``zero_tail`` is false: then they are left as allocated (the reference pads with ``torch.empty``,
+    models/sparvar/sparse_attn.py:1113-1117; nothing reads them), which saves writing the full-width rows.  Equals
     ``append_local_run(map_inds_counts_across_scales(...))`` of :mod:`lvar_amd.mask_build`
     (models/sparvar/sparse_attn.py:366-421, 1096-1121)."""
     _require(src_indices.dim() == 4, "src_indices must be [B,H,Gs,Ks]")
@@ -495,11 +497,12 @@ def remap_concat_lists(src_indices, src_count: int, cur_q_len: int, cur_k_len: i
         L = loc.shape[1]
     out_len = int(cur_k_len) if out_len is None else int(out_len)
     _require(cnt + L <= out_len, lambda: f"list length {cnt + L} exceeds the output width {out_len}")
-    out = torch.empty((B, H, Gk, out_len), dtype=torch.int32, device=src.device)    # the kernel zeroes the tail
+    out = torch.empty((B, H, Gk, out_len), dtype=torch.int32, device=src.device)    # the kernel zeroes the tail (zero_tail)
     counts = torch.empty((B, H, Gk), dtype=torch.int32, device=src.device)
     with _on_device(src):
         st = _lib.load().lvar_remap_concat_lists(src.data_ptr(), Ks, Ks, _ptr(loc), L, L, out.data_ptr(), out_len,
-                                                counts.data_ptr(), B * H, Gs, Gk, cnt, int(cur_k_len), out_len, _stream(src))
+                                                counts.data_ptr(), B * H, Gs, Gk, cnt, int(cur_k_len),
+                                                out_len if zero_tail else cnt + L, _stream(src))
     _lib.check(st, "lvar_remap_concat_lists")
     return out, counts
 

@@ -77,8 +77,9 @@ class SparseDiffAttn(torch.nn.Module):
             local_inds = local_inds.to(inds.device)
             self.local_inds[scale_ind] = (local_inds, local_count)
         # group remap + clamp + local-run append + counts in one launch (sparse_attn.py:1056-1121)
+        # (columns behind the list stay as allocated, as the reference's torch.empty padding, sparse_attn.py:1113-1117)
         inds, counts = ops.remap_concat_lists(inds, s_count, q.shape[-2], k.shape[-2], local_inds,
-                                              bm=self.bm, indices_pad_to=self.indices_pad_to)
+                                              bm=self.bm, indices_pad_to=self.indices_pad_to, zero_tail=False)
         assert int(inds.shape[-1]) >= s_count + local_count and (s_count + local_count) % self.multiple_of == 0, \
             f"after add local sparse index, mismatch multiple_of={self.multiple_of}"
         if scale_ind != len(self.scales) - 1:
