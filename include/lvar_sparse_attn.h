@@ -261,8 +261,9 @@ int lvar_block_topk_lists(const float* block_scores, const uint8_t* base_mask,
  * idx_row_stride >= k; columns [k, zero_to) are set to 0, zero_to <= idx_row_stride, the rest is left untouched)
  * and, if counts is not NULL, k to counts[row].
  * Ties at the k-th value go to the smaller column, so the selected SET equals that of a stable
- * descending sort and is a pure function of the scores.  Radix select, no sort: the rows are read
- * five times from L2.  Replaces `torch.topk(bs, k=indices_count, dim=-1).indices` of the full step
+ * descending sort and is a pure function of the scores (-0.0 and +0.0 tie; NaN scores are not supported).
+ * Radix select, no sort: rows of up to 16384 columns are read once and held in registers, longer ones
+ * are re-read from L2 in every pass.  Replaces `torch.topk(bs, k=indices_count, dim=-1).indices` of the full step
  * (models/sparvar/sparse_attn.py:1012-1036), which returns the same set ordered by value, and the
  * reference's unused quantile kernel (kernels/chipmunk/csrc/indexed_io/topk_indices.cu:26-145).
  */

@@ -22,11 +22,13 @@ __device__ __forceinline__ int lanes_below(unsigned long long bal, int lane) {
 // Exact top-k per row by radix select.  One 512-thread workgroup per row; wave w owns the w-th
 // contiguous eighth of the (padded) row and every thread keeps its KPT keys in registers (KPT = 0:
 // rows too long for that are re-read from L2 in every pass).
-//   up to 3 histogram passes (11 bits each, most significant first, starting below the bits that all
-//   keys of the row share; LDS atomics) narrow the k-th largest key down to its exact value T and the
-//   number `need` of keys equal to T that belong to the selection (ties go to the smaller column);
+//   a histogram pass (11 bits, starting below the bits that all keys of the row share; LDS atomics)
+//   finds the bin of the k-th largest key; the keys of that bin are compared with each other directly
+//   (or, if they are too many, go through up to two more histogram passes), which gives the exact
+//   value T of the k-th largest key and the number `need` of keys equal to T that belong to the
+//   selection (ties go to the smaller column);
 //   a counting pass gives every wave its number of selected keys, the last pass writes the selected
-//   columns in ascending order (ballot compaction).
+//   columns in ascending order (ballot compaction into an LDS ring, full-width stores).
 // ---------------------------------------------------------------------------------------------
 constexpr int TOPK_BINS = 2048;
 constexpr int TOPK_CAND = 256;   // keys of the first pass's bin that are resolved by direct comparison
