@@ -57,6 +57,20 @@ __device__ __forceinline__ bf16x8 pack8(float a0, float a1, float a2, float a3, 
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __builtin_bit_cast(float, u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xffff0000u); }
 
+// Order-preserving map float -> uint32 (larger float <=> larger key); -0.0 and +0.0 get the same key (adding +0.0
+// turns -0.0 into +0.0 and changes nothing else), so that they tie as they do in a comparison of the values.
+__device__ __forceinline__ uint32_t sort_key(float x) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, x + 0.0f);
+  return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+}
+
+// Key of a real entry in the selection kernels: never 0, which is kept for entries that do not compete (padding
+// columns, always-on blocks).  Only a NaN with every bit set maps to 0; it is lifted to 1.
+__device__ __forceinline__ uint32_t real_key(float x) {
+  const uint32_t k = sort_key(x);
+  return k > 1u ? k : 1u;
+}
+
 // Transposing LDS read: the 16 lanes of a group each point at 4 consecutive bf16 of a row;
 // lane i of the group receives element (i%4) of the rows addressed by lanes (i/4), (i/4)+4,
 // (i/4)+8, (i/4)+12.  With lane s addressing row (s/4), columns 4*(s%4)..+3 of a 4x16 block,

@@ -7,13 +7,6 @@
 
 namespace lvar {
 
-// Order-preserving map float -> uint32 (larger float <=> larger key); -0.0 and +0.0 get the same key (adding +0.0
-// turns -0.0 into +0.0 and changes nothing else), so that they tie as they do in a comparison of the values.
-__device__ __forceinline__ uint32_t sort_key(float x) {
-  const uint32_t u = __builtin_bit_cast(uint32_t, x + 0.0f);
-  return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
-}
-
 __device__ __forceinline__ int lanes_below(unsigned long long bal, int lane) {
   return __builtin_popcountll(bal & ((1ull << lane) - 1ull));
 }
@@ -32,11 +25,6 @@ __device__ __forceinline__ int lanes_below(unsigned long long bal, int lane) {
 // ---------------------------------------------------------------------------------------------
 constexpr int TOPK_BINS = 2048;
 constexpr int TOPK_CAND = 256;   // keys of the first pass's bin that are resolved by direct comparison
-
-// Key of a real column: never 0, which is the key of the padding columns beyond the row.  (Only a NaN with every
-// bit set maps to 0; it is lifted to 1.)  Padding keys are then below every real key: they never compare greater than
-// or equal to the threshold, and a histogram counts them at the very bottom, below the k real keys that are wanted.
-__device__ __forceinline__ uint32_t real_key(float x) { return max(sort_key(x), 1u); }
 
 template <int KPT, int NT>
 __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kernel(const TopkListParams p) {
