@@ -270,40 +270,75 @@ int launch_remap_concat_lists(const RemapListParams& p, hipStream_t stream) {
 
 // ---------------------------------------------------------------------------------------------
 // Mask compaction: ascending columns of the set entries of a uint8 row, count rounded up to a
-// multiple with the lowest unset columns as padding.  One wave per row.
+// multiple with the lowest unset columns as padding.  One 256-thread workgroup per row: every wave
+// owns a contiguous quarter of the 64-column chunks, counts its set entries (mask bytes loaded eight
+// chunks at a time), learns its output offset from the counts of the waves before it, and writes
+// its columns on a second sweep; wave 0 then appends the padding.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void mask_to_lists_kernel(const MaskCompactParams p) {
-  const int row = blockIdx.x, lane = threadIdx.x;
+constexpr int MASKLIST_T = 256;
+
+__global__ __launch_bounds__(MASKLIST_T) void mask_to_lists_kernel(const MaskCompactParams p) {
+  constexpr int NW = MASKLIST_T / 64, UN = 8;
+  __shared__ int wcnt[NW];
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint8_t* m = p.mask + (int64_t)row * p.mask_stride;
   int32_t* out = p.indices + (int64_t)row * p.out_stride;
-  const int chunks = (p.n + 63) >> 6;
-  int total = 0;
-  for (int c = 0; c < chunks; c++) {
-    const int j = c * 64 + lane;
-    const bool on = j < p.n && m[j] != 0;
-    const unsigned long long bal = __builtin_amdgcn_ballot_w64(on);
-    if (on) out[total + lanes_below(bal, lane)] = j;
-    total += __builtin_popcountll(bal);
+  const int n = p.n;
+  const int chunks = (n + 63) >> 6;
+  const int cpw = (chunks + NW - 1) / NW;
+  const int c_lo = min(chunks, wave * cpw), c_hi = min(chunks, c_lo + cpw);
+  // sweep(f): f(first column of the chunk, ballot of the set entries) for every chunk of this wave, ascending
+  auto sweep = [&](auto&& f) {
+    for (int c0 = c_lo; c0 < c_hi; c0 += UN) {
+      uint8_t v[UN];
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int j = (c0 + u) * 64 + lane;
+        v[u] = m[min(j, n - 1)];          // clamped: the load is unconditional, its use is not
+      }
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int j = (c0 + u) * 64 + lane;
+        if (c0 + u < c_hi) f((c0 + u) * 64, __builtin_amdgcn_ballot_w64(j < n && v[u] != 0));
+      }
+    }
+  };
+  int mine = 0;
+  sweep([&](int, unsigned long long bal) { mine += __builtin_popcountll(bal); });
+  if (lane == 0) wcnt[wave] = mine;
+  __syncthreads();
+  int pos = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < NW; w++) {
+    pos += (w < wave) ? wcnt[w] : 0;
+    total += wcnt[w];
   }
+  sweep([&](int col0, unsigned long long bal) {
+    if ((bal >> lane) & 1ull) out[pos + lanes_below(bal, lane)] = col0 + lane;
+    pos += __builtin_popcountll(bal);
+  });
   const int mult = max(1, p.multiple_of);
-  const int padded = min(p.n, (total + mult - 1) / mult * mult);
-  int filled = total;
-  for (int c = 0; c < chunks && filled < padded; c++) {
-    const int j = c * 64 + lane;
-    const bool off = j < p.n && m[j] == 0;
-    const unsigned long long bal = __builtin_amdgcn_ballot_w64(off);
-    const int at = filled + lanes_below(bal, lane);
-    if (off && at < padded) out[at] = j;
-    filled = min(padded, filled + __builtin_popcountll(bal));
+  const int padded = min(n, (total + mult - 1) / mult * mult);
+  if (wave == 0) {
+    // padding: the lowest unset columns, in ascending order (fewer than `multiple_of` of them)
+    int filled = total;
+    for (int c = 0; c < chunks && filled < padded; c++) {
+      const int j = c * 64 + lane;
+      const bool off = j < n && m[j] == 0;
+      const unsigned long long bal = __builtin_amdgcn_ballot_w64(off);
+      const int at = filled + lanes_below(bal, lane);
+      if (off && at < padded) out[at] = j;
+      filled = min(padded, filled + __builtin_popcountll(bal));
+    }
   }
   if (p.zero_tail)
-    for (int t = padded + lane; t < p.out_len; t += 64) out[t] = 0;
-  if (lane == 0) p.counts[row] = padded;
+    for (int t = padded + tid; t < p.out_len; t += MASKLIST_T) out[t] = 0;
+  if (tid == 0) p.counts[row] = padded;
 }
 
 int launch_mask_to_lists(const MaskCompactParams& p, hipStream_t stream) {
   if (p.rows == 0) return LVAR_OK;
-  hipLaunchKernelGGL(mask_to_lists_kernel, dim3(p.rows), dim3(64), 0, stream, p);
+  hipLaunchKernelGGL(mask_to_lists_kernel, dim3(p.rows), dim3(MASKLIST_T), 0, stream, p);
   return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
 }
 

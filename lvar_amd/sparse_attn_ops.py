@@ -517,7 +517,8 @@ def mask_to_lists(mask, multiple_of: int = 1):
     capped at ``n`` (the reference's rounded count can exceed the row)."""
     if not mask.is_cuda:
         raise RuntimeError("mask must live on a HIP device; lvar_amd has no CPU path")
-    m = mask.to(torch.uint8).contiguous()
+    # a bool tensor is one byte per entry with the values 0 / 1: viewed, not converted
+    m = (mask.contiguous().view(torch.uint8) if mask.dtype == torch.bool else mask.ne(0).view(torch.uint8).contiguous())
     n = m.shape[-1]
     rows = m.numel() // n if n else 0
     idx = torch.empty(m.shape, dtype=torch.int32, device=m.device)
