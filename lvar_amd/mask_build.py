@@ -42,11 +42,11 @@ def indices_count(top_keys: float, k_len: int, multiple_of: Optional[int] = None
 
 
 def topk_index_list(bs: torch.Tensor, top_keys: float, multiple_of: Optional[int] = None,
-                    indices_pad_to: Optional[int] = None, order: str = "value") -> Tuple[torch.Tensor, torch.Tensor]:
+                    indices_pad_to: Optional[int] = None, order: str = "value", zero_tail: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
     """Full-step list build (models/sparvar/sparse_attn.py:1012-1036): top-k of the colsum ``bs``
     [B,H,G,Lk] -> ``inds`` int32 [B,H,G,Lk] whose first ``count`` columns are valid, and ``counts``
-    int32 [B,H,G].  Padding columns are zero-filled (the reference leaves them uninitialised; they
-    are never read).  ``order="value"`` lists the keys by descending score as ``torch.topk`` does,
+    int32 [B,H,G].  Padding columns are zero-filled unless ``zero_tail`` is false (the reference leaves them
+    uninitialised, sparse_attn.py:1031-1034; they are never read).  ``order="value"`` lists the keys by descending score as ``torch.topk`` does,
     ``order="index"`` by ascending key (same set; the attention kernels do not depend on the order
     and gather ascending lists faster).  A tensor on a HIP device goes through the radix-select
     kernel (:func:`lvar_amd.sparse_attn_ops.topk_token_lists`, ties to the smaller key)."""
@@ -60,7 +60,7 @@ def topk_index_list(bs: torch.Tensor, top_keys: float, multiple_of: Optional[int
         raise ValueError("order must be 'value' or 'index'")
     if bs.is_cuda:
         from . import sparse_attn_ops as ops
-        return ops.topk_token_lists(bs, cnt, out_len=Lk, order=order)
+        return ops.topk_token_lists(bs, cnt, out_len=Lk, order=order, zero_tail=zero_tail)
     inds = torch.zeros((B, H, G, Lk), dtype=torch.int32, device=bs.device)
     if cnt > 0:
         top = torch.topk(bs, k=cnt, dim=-1).indices

@@ -437,11 +437,12 @@ def block_topk_lists(block_scores, target: int, base_mask=None):
     return num, idx
 
 
-def topk_token_lists(scores, k: int, out_len: Optional[int] = None, order: str = "index"):
+def topk_token_lists(scores, k: int, out_len: Optional[int] = None, order: str = "index", zero_tail: bool = True):
     """Exact top-``k`` key columns of every row of ``scores`` (fp32 ``[..., Lk]``, e.g. the column sums
     ``[B,H,G,Lk]``) on the GPU: returns ``(indices int32 [..., out_len], counts int32 [...])`` with the
     selected columns in the first ``k`` entries (``out_len`` defaults to ``Lk``, the width the list
-    attention op expects; entries beyond ``k`` are zero).  ``order="index"`` (default, one kernel)
+    attention op expects; entries beyond ``k`` are zero, or left as allocated with ``zero_tail=False``: nothing reads
+    them).  ``order="index"`` (default, one kernel)
     lists them in ascending column order, which is also the best order for the gather kernel;
     ``order="value"`` re-orders them by descending score like ``torch.topk``
     (models/sparvar/sparse_attn.py:1016).  Ties at the k-th value go to the smaller column."""
@@ -460,7 +461,7 @@ def topk_token_lists(scores, k: int, out_len: Optional[int] = None, order: str =
     cnt = torch.empty(sc.shape[:-1], dtype=torch.int32, device=sc.device)
     with _on_device(sc):
         st = _lib.load().lvar_topk_token_lists(sc.data_ptr(), Lk, idx.data_ptr(), out_len, cnt.data_ptr(),
-                                              rows, Lk, k, out_len, _stream(sc))
+                                              rows, Lk, k, out_len if zero_tail else k, _stream(sc))
     _lib.check(st, "lvar_topk_token_lists")
     if order == "value" and k > 0:
         sel = idx[..., :k].long()

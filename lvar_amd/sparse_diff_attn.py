@@ -60,7 +60,7 @@ class SparseDiffAttn(torch.nn.Module):
         top_keys = GLOBAL_CONFIG["attn"]["top_keys"]
         if do_full_step:                                           # sparse_attn.py:991-1051
             o, bs = self.dense_colsum_attn(q, k, v, scale)
-            inds, counts = mb.topk_index_list(bs, top_keys, self.multiple_of, self.indices_pad_to, order="index")
+            inds, counts = mb.topk_index_list(bs, top_keys, self.multiple_of, self.indices_pad_to, order="index", zero_tail=False)
             self.indices, self.counts = inds, counts
             self.count_host = mb.indices_count(top_keys, k.shape[-2], self.multiple_of)
             if self.use_o_cache:
