@@ -704,31 +704,74 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
   if (LSE_ONLY) return;
 
   const float osc = ACCUM ? p.o_scale * inv : inv;
-  char* ob = smem + wave * (32 * OSTR);
-  const bf16_t* oap = nullptr;
-  // bilinear taps of this lane's query in a coarser o_accum grid (half-pixel centres, edge clamp:
-  // src = max(0, (dst + 0.5) * src_side / dst_side - 0.5), the align_corners = False rule)
-  const bf16_t *tap01 = nullptr, *tap10 = nullptr, *tap11 = nullptr;
-  float wy1 = 0.f, wx1 = 0.f;
-  if (ACCUM && p.o_accum) {
-    const bf16_t* base = p.o_accum + b * p.oa_sb + h * p.oa_sh;
-    const int qr = min(qrow_w, p.Lq - 1);
-    if (p.up_src > 0) {
-      const int y = qr / p.up_dst, x = qr - y * p.up_dst;
-      const float sc = (float)p.up_src / (float)p.up_dst;
-      const float sy = fmaxf(sc * ((float)y + 0.5f) - 0.5f, 0.f), sx = fmaxf(sc * ((float)x + 0.5f) - 0.5f, 0.f);
-      const int y0 = min((int)sy, p.up_src - 1), x0 = min((int)sx, p.up_src - 1);
-      const int y1 = min(y0 + 1, p.up_src - 1), x1 = min(x0 + 1, p.up_src - 1);
-      wy1 = sy - (float)y0;
-      wx1 = sx - (float)x0;
-      oap = base + (int64_t)(y0 * p.up_src + x0) * p.oa_sr;
-      tap01 = base + (int64_t)(y0 * p.up_src + x1) * p.oa_sr;
-      tap10 = base + (int64_t)(y1 * p.up_src + x0) * p.oa_sr;
-      tap11 = base + (int64_t)(y1 * p.up_src + x1) * p.oa_sr;
-    } else {
-      oap = base + (int64_t)qr * p.oa_sr;
+  if constexpr (ACCUM) {
+    if (p.o_accum) {
+      // o = o_accum (or its bilinear upsample) + o_scale * O / l, formed in fp32 and rounded once.  The accumulators
+      // go through LDS as fp32, half of the head dimension at a time (the K/V buffers hold 32 rows x D/2 floats per
+      // wave), so that a lane ends up with 8 consecutive columns of one row: the o_accum rows (four taps of the
+      // coarser grid when upsampling: half-pixel centres, edge clamp, src = max(0, (dst + 0.5) * src_side / dst_side
+      // - 0.5), the align_corners = False rule) are then read with 16-byte loads that 8 neighbouring lanes share a
+      // row of, and o is stored the same way.
+      constexpr int HD = D / 2, FSTR = HD * 4 + 16, CPRH = HD / 8, ITER = (32 * CPRH) / 64;
+      static_assert(NCOMP * 32 * FSTR <= 4 * TILE, "fp32 epilogue buffer must fit in the K/V buffers");
+      char* fb = smem + wave * (32 * FSTR);
+      const bf16_t* abase = p.o_accum + b * p.oa_sb + h * p.oa_sh;
+      bf16_t* op = p.o + b * p.o_sb + h * p.o_sh;
+#pragma unroll
+      for (int pass = 0; pass < 2; pass++) {
+#pragma unroll
+        for (int mm = 0; mm < MTD / 2; mm++) {
+          const int m = pass * (MTD / 2) + mm;
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            const f32x4 x = {oacc[m][4 * a + 0] * osc, oacc[m][4 * a + 1] * osc, oacc[m][4 * a + 2] * osc, oacc[m][4 * a + 3] * osc};
+            *(f32x4*)(fb + r * FSTR + (mm * 32 + 8 * a + 4 * hh) * 4) = x;
+          }
+        }
+        // each wave re-reads only its own 32 rows: a wave-local fence is enough
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < ITER; i++) {
+          const int cidx = lane + i * 64;
+          const int orow = cidx / CPRH, oc = cidx - orow * CPRH;
+          const int grow = q0 + wave * 32 + orow;
+          if (grow < p.Lq) {
+            const f32x4 xa = *(const f32x4*)(fb + orow * FSTR + oc * 32), xb = *(const f32x4*)(fb + orow * FSTR + oc * 32 + 16);
+            float x[8] = {xa[0], xa[1], xa[2], xa[3], xb[0], xb[1], xb[2], xb[3]};
+            const int col = pass * HD + oc * 8;
+            if (p.up_src > 0) {
+              const int y = grow / p.up_dst, xq = grow - y * p.up_dst;
+              const float sc = (float)p.up_src / (float)p.up_dst;
+              const float sy = fmaxf(sc * ((float)y + 0.5f) - 0.5f, 0.f), sx = fmaxf(sc * ((float)xq + 0.5f) - 0.5f, 0.f);
+              const int y0 = min((int)sy, p.up_src - 1), x0 = min((int)sx, p.up_src - 1);
+              const int y1 = min(y0 + 1, p.up_src - 1), x1 = min(x0 + 1, p.up_src - 1);
+              const float wy1 = sy - (float)y0, wx1 = sx - (float)x0, wy0 = 1.f - wy1, wx0 = 1.f - wx1;
+              const u32x4 t00 = *(const u32x4*)(abase + (int64_t)(y0 * p.up_src + x0) * p.oa_sr + col);
+              const u32x4 t01 = *(const u32x4*)(abase + (int64_t)(y0 * p.up_src + x1) * p.oa_sr + col);
+              const u32x4 t10 = *(const u32x4*)(abase + (int64_t)(y1 * p.up_src + x0) * p.oa_sr + col);
+              const u32x4 t11 = *(const u32x4*)(abase + (int64_t)(y1 * p.up_src + x1) * p.oa_sr + col);
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                x[2 * e] += wy0 * (wx0 * bf16_lo(t00[e]) + wx1 * bf16_lo(t01[e])) + wy1 * (wx0 * bf16_lo(t10[e]) + wx1 * bf16_lo(t11[e]));
+                x[2 * e + 1] += wy0 * (wx0 * bf16_hi(t00[e]) + wx1 * bf16_hi(t01[e])) + wy1 * (wx0 * bf16_hi(t10[e]) + wx1 * bf16_hi(t11[e]));
+              }
+            } else {
+              const u32x4 t = *(const u32x4*)(abase + (int64_t)grow * p.oa_sr + col);
+#pragma unroll
+              for (int e = 0; e < 4; e++) { x[2 * e] += bf16_lo(t[e]); x[2 * e + 1] += bf16_hi(t[e]); }
+            }
+            const u32x4 val = {pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7])};
+            *(u32x4*)(op + (int64_t)grow * p.o_sr + col) = val;
+          }
+        }
+        __builtin_amdgcn_wave_barrier();   // the buffer is rewritten by the next pass
+      }
+      return;
     }
   }
+  char* ob = smem + wave * (32 * OSTR);
 #pragma unroll
   for (int m = 0; m < MTD; m++) {
 #pragma unroll
@@ -736,19 +779,6 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       const int dcol = m * 32 + 8 * a + 4 * hh;
       float x0 = oacc[m][4 * a + 0] * osc, x1 = oacc[m][4 * a + 1] * osc;
       float x2 = oacc[m][4 * a + 2] * osc, x3 = oacc[m][4 * a + 3] * osc;
-      if (ACCUM && oap) {
-        u32x2 acc = *(const u32x2*)(oap + dcol);
-        float a0 = bf16_lo(acc[0]), a1 = bf16_hi(acc[0]), a2 = bf16_lo(acc[1]), a3 = bf16_hi(acc[1]);
-        if (tap01) {
-          const u32x2 t01 = *(const u32x2*)(tap01 + dcol), t10 = *(const u32x2*)(tap10 + dcol), t11 = *(const u32x2*)(tap11 + dcol);
-          const float wy0 = 1.f - wy1, wx0 = 1.f - wx1;
-          a0 = wy0 * (wx0 * a0 + wx1 * bf16_lo(t01[0])) + wy1 * (wx0 * bf16_lo(t10[0]) + wx1 * bf16_lo(t11[0]));
-          a1 = wy0 * (wx0 * a1 + wx1 * bf16_hi(t01[0])) + wy1 * (wx0 * bf16_hi(t10[0]) + wx1 * bf16_hi(t11[0]));
-          a2 = wy0 * (wx0 * a2 + wx1 * bf16_lo(t01[1])) + wy1 * (wx0 * bf16_lo(t10[1]) + wx1 * bf16_lo(t11[1]));
-          a3 = wy0 * (wx0 * a3 + wx1 * bf16_hi(t01[1])) + wy1 * (wx0 * bf16_hi(t10[1]) + wx1 * bf16_hi(t11[1]));
-        }
-        x0 += a0; x1 += a1; x2 += a2; x3 += a3;
-      }
       u32x2 pk = {pack_bf16(x0, x1), pack_bf16(x2, x3)};
       *(u32x2*)(ob + r * OSTR + dcol * 2) = pk;
     }
