@@ -61,7 +61,7 @@ typedef struct {
 } lvar_workspace_t;
 
 /* Bytes of a workspace that lets every balanced launch of the current device use all its slots
- * (head_dim 64 or 128), or a negative LVAR_E* code. */
+ * (head_dim 64 or 128; head_dim 256 has no balanced launch: LVAR_EUNSUPPORTED), or a negative LVAR_E* code. */
 int64_t lvar_attn_workspace_bytes(int head_dim);
 
 /* Workgroups a *_ws_fwd launch of these sizes would run as a balanced launch on the current device, 0 if it
@@ -82,7 +82,10 @@ const char* lvar_status_string(int status);
  * (kernels/sparse_attn/triton/attn_dense.py:186-231).
  * LSE2, if not NULL, receives the base-2 log-sum-exp M + log2(L) (fp32 [B,H,Lq]), the form the
  * colsum entry point consumes.  o may be NULL (statistics only); M, L and LSE2 may each be NULL.
- * head_dim in {64, 128}.  Grouped-query attention: k and v hold kv_heads heads, H a multiple of it, and query
+ * head_dim in {64, 128, 256} (256: one wave per SIMD with 512 registers and 128 KiB of LDS per workgroup, always
+ * the plain launch; built for coverage of the reference's Triton range, kernels/sparse_attn/triton/
+ * attn_dense_colsum.py:246, not tuned).  This holds for every attention, colsum and window-score entry point
+ * below except the static-scratch one.  Grouped-query attention: k and v hold kv_heads heads, H a multiple of it, and query
  * head h reads K/V head h / (H / kv_heads) (the layout of the reference's expansion, kernels/sparse_attn/
  * sparse_attn_ops.py:228-233; kernels/chipmunk/csrc/attn/dense_colsum_attn.cu:386-387); kv_heads = H otherwise.
  */

@@ -64,10 +64,13 @@ struct Swz {
   static constexpr int ROWB = D * 2;      // bytes per K/V row
   static constexpr int CPR = ROWB / 16;   // 16-byte chunks per row
   // chunk-index XOR of the K tile: makes ds_read_b128 of 16 consecutive rows conflict-free
-  __device__ static __forceinline__ int fk(int row) { return (row / (256 / ROWB)) & (CPR - 1); }
+  // (rows of 256 bytes or more: the row index itself, 16 rows per period)
+  __device__ static __forceinline__ int fk(int row) {
+    if constexpr (ROWB >= 256) return row & 15; else return (row / (256 / ROWB)) & (CPR - 1);
+  }
   // chunk-index XOR of the V tile: moves the 64-byte segment read by the transposing loads of
   // 4 consecutive rows onto 4 different bank groups
-  __device__ static __forceinline__ int fv(int row) { return (D == 128) ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+  __device__ static __forceinline__ int fv(int row) { return (D >= 128) ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 };
 
 // Context of a balanced launch (see sk_partition.h); unused by the plain launch.
@@ -97,6 +100,9 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
   constexpr int NI = 64 / RPI;              // loads per 64-row tile
   constexpr int SLOTS = (NI + FW - 1) / FW;
   constexpr int TILE = 64 * ROWB;
+  // block lists: the rows of a tile are consecutive, so a fill's lane offset can be a constant (see issue_slot)
+  constexpr bool CONST_OFF = MODE == MODE_BLOCK && ((FW * RPI) % 16 == 0 || 16 % (FW * RPI) == 0) && NI % FW == 0;
+  constexpr int CONST_PER = (FW * RPI) >= 16 ? 1 : 16 / (FW * RPI);
   constexpr int OSTR = D * 2 + 16;  // epilogue transpose buffer row stride (bytes)
   static_assert(NCOMP * 32 * OSTR <= 4 * TILE, "epilogue buffer must fit in the K/V buffers");
   // LDS map: K buffers at 0 and TILE, V buffers at 2*TILE and 3*TILE
@@ -212,12 +218,13 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       // slot) is a constant and tile and slot only move a scalar offset.
       // The buffer descriptor ends with the last key row, so the rows of a ragged last tile that lie beyond it read
       // as zeros (they are masked in the softmax); the first row is never negative (finish_rows clamps the block).
-      // (Needs the slots of one wave a swizzle period, 16 rows, apart: not so for two waves at head_dim 128.)
-      if constexpr (MODE == MODE_BLOCK && (FW * RPI) % 16 == 0) {
+      // (The swizzle has a period of 16 rows: slots whose rows are a whole period apart share the lane offset.  When
+      // the FW * RPI rows that the filling waves cover per slot are fewer than 16, CONST_PER such offsets alternate.)
+      if constexpr (CONST_OFF) {
         const int row0 = __builtin_amdgcn_readfirstlane(rows[0]);  // wave-uniform for block lists
-        const int trow0 = fwave * RPI + lrow;
+        const int trow0 = (fwave + (s % CONST_PER) * FW) * RPI + lrow;
         const int voff = trow0 * srb + ((lcs ^ (is_v ? Swz<D>::fv(trow0) : Swz<D>::fk(trow0))) << 4);
-        const int soff = (row0 + s * FW * RPI) * srb;
+        const int soff = (row0 + (s / CONST_PER) * CONST_PER * FW * RPI) * srb;
         asm volatile(
             "s_mov_b32 m0, %0\n\t"
             "s_nop 0\n\t"
@@ -436,7 +443,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       // shadow of the MFMA before.  NFILL instructions, one every FSTRIDE steps; if there are more than steps, up front.
       constexpr int NQK_ = 2 * KS;
       constexpr int NFILL = NPROD ? 0 : (LSE_ONLY ? SLOTS : 2 * SLOTS);
-      constexpr int FSTRIDE = (MODE == MODE_BLOCK && (FW * RPI) % 16 == 0 && NFILL > 0 && NFILL <= NQK_) ? NQK_ / NFILL : 0;
+      constexpr int FSTRIDE = (CONST_OFF && NFILL > 0 && NFILL <= NQK_) ? NQK_ / NFILL : 0;
       const bool fill_k = t + 2 < T;
       auto fill_step = [&](auto jc) {
         constexpr int j = decltype(jc)::value;
@@ -803,7 +810,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
 #endif  // __HIP_DEVICE_COMPILE__
 
 template <int D, int NWAVES, int MODE, bool ACCUM, bool LSE_ONLY>
-__global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_kernel(const AttnParams p) {
+__global__ __launch_bounds__(NWAVES * 64, ((NWAVES <= 4 && D <= 128) ? 2 : 1)) void attn_fwd_kernel(const AttnParams p) {
   // The body is compiled for the device only: the host pass just needs the launch stub, and it
   // silently drops the stub when the body uses the LDS-DMA builtins.
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -954,7 +961,7 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
     const int64_t per_tile = (MODE == MODE_BLOCK) ? (p.list ? p.list_len : (p.Lk + 63) / 64) : (p.list_len + 63) / 64;
     const int sub = (MODE == MODE_BLOCK && p.list) ? p.sub_shift : 0;
     // (64-row query blocks always take the plain launch)
-    p.sk_wgs = (p.sk_ws && NWAVES != 2) ? sk_plan(p.total_wg, NWAVES, sk_slot_floats(D, MODE, NWAVES), per_tile, sub, p.sk_ws_bytes,
+    p.sk_wgs = (p.sk_ws && NWAVES != 2 && D <= 128) ? sk_plan(p.total_wg, NWAVES, sk_slot_floats(D, MODE, NWAVES), per_tile, sub, p.sk_ws_bytes,
                                  p.sk_min_share, p.sk_min_piece) : 0;
     p.sk_uniform_n = 0;
     if (p.sk_wgs > 0 && dense) {
@@ -964,7 +971,7 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
       const int n = sk_worth_cutting(U, S, p.total_wg, p.sk_wgs) ? sk_pieces(T, S, p.sk_min_piece) : 1;
       if (n > 1 && (int64_t)n * p.total_wg <= 2 * p.sk_wgs) p.sk_uniform_n = n; else p.sk_wgs = 0;   // whole tiles: the plain launch
     }
-    if constexpr (NWAVES != 2) if (p.sk_wgs > 0) {
+    if constexpr (NWAVES != 2 && D <= 128) if (p.sk_wgs > 0) {
       p.sk_counters = (int*)p.sk_ws;
       p.sk_slots = (float*)((char*)p.sk_ws + SK_COUNTER_BYTES + sk_plan_bytes(p.sk_wgs));
       int grid_sk;
@@ -1002,7 +1009,9 @@ static int launch_d(const AttnParams& p, int mode, bool accum, bool lse_only, in
     if (nwaves != 4) return LVAR_EUNSUPPORTED;
     return lse_only ? launch_one<D, 4, MODE_BLOCK, false, true>(p, s) : launch_one<D, 4, MODE_BLOCK, false, false>(p, s);
   } else if (mode == MODE_GATHER) {
-    if (nwaves == 8) return launch_one<D, 8, MODE_GATHER, true, false>(p, s);
+    // (head_dim 256: a wave needs more than 256 registers, so one wave per SIMD: 192-row groups run as two 3-wave workgroups)
+    if constexpr (D > 128) { if (nwaves == 8) nwaves = 3; }
+    else if (nwaves == 8) return launch_one<D, 8, MODE_GATHER, true, false>(p, s);
     if (nwaves == 3) return launch_one<D, 3, MODE_GATHER, true, false>(p, s);
     if (nwaves == 2) return launch_one<D, 2, MODE_GATHER, true, false>(p, s);
   }
@@ -1012,6 +1021,7 @@ static int launch_d(const AttnParams& p, int mode, bool accum, bool lse_only, in
 int launch_attn(const AttnParams& p, int head_dim, int mode, bool accum, bool lse_only, int nwaves, hipStream_t s) {
   if (head_dim == 128) return launch_d<128>(p, mode, accum, lse_only, nwaves, s);
   if (head_dim == 64) return launch_d<64>(p, mode, accum, lse_only, nwaves, s);
+  if (head_dim == 256) return launch_d<256>(p, mode, accum, lse_only, nwaves, s);
   return LVAR_EUNSUPPORTED;
 }
 

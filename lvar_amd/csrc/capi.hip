@@ -271,8 +271,8 @@ int lvar_block_sparse_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_
 
 int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, int H, int Lq, int Lk, int list_len,
                                   int head_dim, lvar_workspace_t workspace) {
-  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || (head_dim != 64 && head_dim != 128) || kind < 0 || kind > 2) return LVAR_EINVAL;
-  if (!workspace.ptr) return 0;
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || (head_dim != 64 && head_dim != 128 && head_dim != 256) || kind < 0 || kind > 2) return LVAR_EINVAL;
+  if (!workspace.ptr || head_dim == 256) return 0;   // head_dim 256 always takes the plain launch
   int nwaves = 4, mode = MODE_BLOCK, sub = 0;
   int64_t per_tile = (Lk + 63) / 64;
   if (kind == 1) {

@@ -19,11 +19,13 @@
 namespace lvar {
 
 template <int D>
-__global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
+__global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void colsum_kernel(const ColsumParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int KS = D / 16;
   constexpr int ROWB = D * 2, CPR = ROWB / 16;
   constexpr int RPI = 1024 / ROWB, NI = 64 / RPI, SLOTS = NI / 4;
+  constexpr int SWD = ROWB >= 256 ? 1 : 256 / ROWB;   // chunk swizzle of row t: (t / SWD) & SWM, 16 rows per period
+  constexpr int SWM = ROWB >= 256 ? 15 : CPR - 1;
   constexpr int QTILE = 64 * ROWB;         // one 64-row Q stage
   constexpr int NSTAGE = 4, NLSE = 8;      // ring depths
   constexpr int LSE_OFF = NSTAGE * QTILE;  // lse2 ring: NLSE x 64 floats
@@ -71,12 +73,17 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
   const int lrow = lane / CPR, lcs = lane % CPR;
 
   // global->LDS fill of stage s (Q rows s*64 .. +63, clamped to Lq-1, chunk-swizzled; lse2 by wave 0)
-  // lane offset of a Q fill: row within the first instruction of this wave, swizzled chunk (the swizzle
-  // repeats every 16 rows, i.e. does not depend on the slot: instruction i = wave + 4 * slot covers rows
-  // i * RPI ..)
-  static_assert((4 * RPI) % 16 == 0, "slots of one wave must be a swizzle period (16 rows) apart");
-  const int fill_trow0 = wave * RPI + lrow;
-  const int fill_voff = fill_trow0 * q_srb + ((lcs ^ ((fill_trow0 / (256 / ROWB)) & (CPR - 1))) << 4);
+  // lane offset of a Q fill: row within the first instruction(s) of this wave, swizzled chunk.  The swizzle
+  // repeats every 16 rows and instruction i = wave + 4 * slot covers rows i * RPI ..: slots a whole period apart
+  // share the lane offset (PER = 1: all of them; head_dim 256 has two rows per instruction and PER = 2).
+  constexpr int PER = (4 * RPI >= 16) ? 1 : 16 / (4 * RPI);
+  static_assert((PER * 4 * RPI) % 16 == 0 && SLOTS % PER == 0, "slots PER apart must be whole swizzle periods apart");
+  int fill_voff[PER];
+#pragma unroll
+  for (int ph = 0; ph < PER; ph++) {
+    const int trow = (wave + 4 * ph) * RPI + lrow;
+    fill_voff[ph] = trow * q_srb + ((lcs ^ ((trow / SWD) & SWM)) << 4);
+  }
   auto issue_stage = [&](int s) {
     const uint32_t dst = lds0 + (s & (NSTAGE - 1)) * QTILE;
     if (s * 64 + 64 <= Lq_l) {
@@ -84,9 +91,9 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
 #pragma unroll
       for (int sl = 0; sl < SLOTS; sl++) {
         const int i = wave + sl * 4;
-        const int soff = (qoff + s * 64 + sl * 4 * RPI) * q_srb;
+        const int soff = (qoff + s * 64 + (sl / PER) * PER * 4 * RPI) * q_srb;
         const uint32_t m0v = dst + i * 1024;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(m0v), "v"(fill_voff), "s"(qrsrc), "s"(soff) : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(m0v), "v"(fill_voff[sl % PER]), "s"(qrsrc), "s"(soff) : "memory");
       }
     } else {
 #pragma unroll
@@ -94,7 +101,7 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
         const int i = wave + sl * 4;
         const int trow = i * RPI + lrow;
         const int grow = min(qoff + s * 64 + trow, p.Lq - 1);
-        const int voff = grow * q_srb + ((lcs ^ ((trow / (256 / ROWB)) & (CPR - 1))) << 4);
+        const int voff = grow * q_srb + ((lcs ^ ((trow / SWD) & SWM)) << 4);
         const uint32_t m0v = dst + i * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(m0v), "v"(voff), "s"(qrsrc) : "memory");
       }
@@ -106,11 +113,13 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
     }
   };
   // wait until at most `younger` later stages of this wave's fills are still in flight
+  // (s_waitcnt immediate: vmcnt is split into bits 3:0 and 15:14; expcnt and lgkmcnt stay at "don't wait")
+  constexpr auto vm = [](int n) constexpr { return 0x0f70 | (n & 15) | (((n >> 4) & 3) << 14); };
   auto wait_fills = [&](int younger) {
     if (younger >= 2) {
-      if (wave == 0) __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * (SLOTS + 1))); else __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * SLOTS));
+      if (wave == 0) __builtin_amdgcn_s_waitcnt(vm(2 * (SLOTS + 1))); else __builtin_amdgcn_s_waitcnt(vm(2 * SLOTS));
     } else if (younger == 1) {
-      if (wave == 0) __builtin_amdgcn_s_waitcnt(0x0f70 | (SLOTS + 1)); else __builtin_amdgcn_s_waitcnt(0x0f70 | SLOTS);
+      if (wave == 0) __builtin_amdgcn_s_waitcnt(vm(SLOTS + 1)); else __builtin_amdgcn_s_waitcnt(vm(SLOTS));
     } else {
       __builtin_amdgcn_s_waitcnt(0x0f70);
     }
@@ -139,7 +148,7 @@ __global__ __launch_bounds__(256, 2) void colsum_kernel(const ColsumParams p) {
 
   const int S = (Lq_l + 63) >> 6;          // stages of this range
   const int U = (Lq_l + 31) >> 5;          // 32-row tiles
-  const int kbase_l = r * ROWB + ((hh ^ ((r / (256 / ROWB)) & (CPR - 1))) << 4);
+  const int kbase_l = r * ROWB + ((hh ^ ((r / SWD) & SWM)) << 4);
   float acc[2] = {0.f, 0.f};
 
   // probabilities of tile u from its logits: p = exp2(s*c - lse2[row]); rows >= Lq add nothing
@@ -299,6 +308,7 @@ static int launch_cs(const ColsumParams& p0, hipStream_t stream) {
 int launch_colsum(const ColsumParams& p, int head_dim, hipStream_t s) {
   if (head_dim == 128) return launch_cs<128>(p, s);
   if (head_dim == 64) return launch_cs<64>(p, s);
+  if (head_dim == 256) return launch_cs<256>(p, s);
   return LVAR_EUNSUPPORTED;
 }
 

@@ -118,6 +118,7 @@ int launch_window_scores(const WinScoreParams& p0, int head_dim, hipStream_t str
   const dim3 grid(p.B * p.H * p.nchunks);
   if (head_dim == 128) hipLaunchKernelGGL(window_scores_kernel<128>, grid, dim3(256), 0, stream, p);
   else if (head_dim == 64) hipLaunchKernelGGL(window_scores_kernel<64>, grid, dim3(256), 0, stream, p);
+  else if (head_dim == 256) hipLaunchKernelGGL(window_scores_kernel<256>, grid, dim3(256), 0, stream, p);
   else return LVAR_EUNSUPPORTED;
   return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
 }

@@ -91,8 +91,8 @@ def _check_qkv(q, k, v, gqa: bool = False):
     if qs[0] != ks[0] or qs[3] != ks[3] or (qs[1] != ks[1] and not (gqa and ks[1] > 0 and qs[1] % ks[1] == 0)):
         raise ShapeError(f"q/k batch, head or head_dim mismatch: {tuple(q.shape)} vs {tuple(k.shape)}"
                          + ("" if gqa or qs[1] == ks[1] else " (this op takes as many K/V heads as query heads)"))
-    if qs[3] != 128 and qs[3] != 64:
-        raise ShapeError(f"head_dim must be 16, 32, 64 or 128, got {q.shape[-1]}")
+    if qs[3] != 128 and qs[3] != 64 and qs[3] != 256:
+        raise ShapeError(f"head_dim must be 16, 32, 64, 128 or 256, got {q.shape[-1]}")
     if not (q.device == k.device == v.device):
         raise ShapeError("q, k, v must be on the same device")
 

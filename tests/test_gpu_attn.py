@@ -419,4 +419,39 @@ def test_small_head_dims_by_zero_padding(d):
     ob, _ = ops.block_sparse_attn(qg, kg, vg, num.cuda(), idx.cuda(), 128, 64)
     check_o(ob, oracle.block_sparse_attn(q, k, v, num, idx, 128, 64)[0], "block small d")
     with pytest.raises(AssertionError):
-        ops.dense_attn(*dev(*make_qkv(1, 1, 8, 8, 256, seed=1)))
+        ops.dense_attn(*dev(*make_qkv(1, 1, 8, 8, 512, seed=1)))
+
+
+def test_head_dim_256():
+    """head_dim 256, the top of the range the reference's Triton kernels take (attn_dense_colsum.py:246): every
+    operator of the path, ragged sizes, against the oracle."""
+    from lvar_amd import mask_build as mb, sparse_attn_ops as ops
+    d = 256
+    for (B, H, Lq, Lk) in [(1, 2, 300, 1000), (2, 3, 33, 25), (1, 1, 1, 1), (1, 2, 520, 2100)]:
+        q, k, v = make_qkv(B, H, Lq, Lk, d, seed=Lq + Lk)
+        o_ref, M_ref, L_ref = oracle.dense_attn(q, k, v)
+        o, (M, L) = ops.dense_attn(*dev(q, k, v))
+        check_o(o, o_ref, f"dense d=256 {Lq}x{Lk}")
+        check_lse(M, L, M_ref, L_ref)
+    B, H, Lq, Lk = 1, 2, 520, 2100
+    qg, kg, vg = dev(q, k, v)
+    # colsum next to the dense pass
+    o2, cs, _ = ops.dense_colsum_attn(qg, kg, vg)
+    _, cs_ref, _ = oracle.dense_colsum_attn(q, k, v)
+    assert torch.equal(o2, o) and torch.allclose(cs.cpu(), cs_ref, rtol=1e-3, atol=1e-6)
+    # token lists: 192-row groups (two 3-wave workgroups per group), cache delta
+    inds, counts = mb.topk_index_list(cs, 0.3)
+    out = ops.csp_attn(qg, kg, vg, 0.3, inds, counts, o, -1)
+    check_o(out, oracle.csp_attn(q, k, v, 0.3, inds.cpu(), counts.cpu(), o.cpu(), -1), "csp d=256")
+    # block lists: 128-row and 64-row query blocks, 64- and 128-key blocks
+    for bq, bk in [(128, 64), (64, 64), (128, 128)]:
+        nq, nk = (Lq + bq - 1) // bq, (Lk + bk - 1) // bk
+        mask = torch.rand(B, H, nq, nk, generator=torch.Generator().manual_seed(bq + bk)) < 0.4
+        mask[0, 0, 1] = False    # an empty list
+        num, idx = oracle.block_mask_to_lists(mask)
+        ob, _ = ops.block_sparse_attn(qg, kg, vg, num.cuda(), idx.cuda(), bq, bk)
+        check_o(ob, oracle.block_sparse_attn(q, k, v, num, idx, bq, bk)[0], f"block d=256 {bq}x{bk}")
+    # grouped-query attention
+    kq, vq = k[:, :1].contiguous(), v[:, :1].contiguous()
+    og, _ = ops.dense_attn(qg, kq.cuda(), vq.cuda())
+    check_o(og, oracle.dense_attn(q, kq.expand(-1, H, -1, -1), vq.expand(-1, H, -1, -1))[0], "gqa d=256")

@@ -330,7 +330,8 @@ def test_window_key_scores_and_scalekv_selection():
     from lvar_amd import sparse_attn_ops as ops
     g = torch.Generator().manual_seed(15)
     for (B, H, Lq, Lk, d, W, ks, pooling) in ((1, 2, 400, 921, 128, 16, 5, "avgpool"), (2, 3, 64, 700, 64, 9, 7, "maxpool"),
-                                              (1, 1, 300, 300, 128, 4, 1, "avgpool"), (1, 2, 1024, 2521, 128, 256, 5, "maxpool")):
+                                              (1, 1, 300, 300, 128, 4, 1, "avgpool"), (1, 2, 1024, 2521, 128, 256, 5, "maxpool"),
+                                              (1, 2, 200, 1300, 256, 24, 3, "avgpool")):
         q = (torch.randn(B, H, Lq, d, generator=g) * 0.5).to(torch.bfloat16)
         k = (torch.randn(B, H, Lk, d, generator=g) * 0.5).to(torch.bfloat16)
         win = torch.randint(Lk - Lq, Lk, (B, H, W), generator=g)
