@@ -94,6 +94,39 @@ def test_token_lists_random(seed):
     assert close(delta, d_ref) and lse_close(M, L, M_ref, L_ref)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_head_dim_256_random(seed):
+    """The three attention forms and the colsum at head_dim 256 on random ragged shapes, strided storage included."""
+    from lvar_amd import sparse_attn_ops as ops
+    g = torch.Generator().manual_seed(4000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    B, H, d = r(1, 2), r(1, 2), 256
+    Lq, Lk = r(1, 500), r(1, 900)
+    scale = (None, 0.05)[r(0, 1)]
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=seed, amp=(0.3, 0.7)[r(0, 1)])
+    mode = r(0, 2)
+    qg, kg, vg = strided(q, mode), strided(k, mode), strided(v, mode)
+    o, (M, L) = ops.dense_attn(qg, kg, vg, scale)
+    o_ref, M_ref, L_ref = oracle.dense_attn(q, k, v, scale)
+    assert close(o, o_ref) and lse_close(M, L, M_ref, L_ref), (B, H, Lq, Lk, scale, mode)
+    grp = (32, 64, 128, 192)[r(0, 3)]
+    cs = ops.colsum(qg, kg, scale, q_group_size=grp)
+    _, cs_ref, _ = oracle.dense_colsum_attn(q, k, v, scale, q_group_size=grp)
+    assert torch.allclose(cs.cpu(), cs_ref, rtol=2e-3, atol=1e-6), (B, H, Lq, Lk, grp)
+    bq, bk = (64, 128, 256)[r(0, 2)], (64, 128, 256)[r(0, 2)]
+    mask = torch.rand(B, H, (Lq + bq - 1) // bq, (Lk + bk - 1) // bk, generator=g) < (0.2, 0.6)[r(0, 1)]
+    num, idx = oracle.block_mask_to_lists(mask)
+    ob, (Mb, Lb) = ops.block_sparse_attn(qg, kg, vg, num.cuda(), idx.cuda(), bq, bk, scale)
+    ob_ref, Mb_ref, Lb_ref = oracle.block_sparse_attn(q, k, v, num, idx, bq, bk, scale)
+    assert close(ob, ob_ref) and lse_close(Mb, Lb, Mb_ref, Lb_ref), (B, H, Lq, Lk, bq, bk)
+    G = (Lq + 191) // 192
+    tidx = torch.randint(0, Lk, (B, H, G, Lk), generator=g, dtype=torch.int32)
+    tcnt = torch.randint(0, Lk + 1, (B, H, G), generator=g, dtype=torch.int32)
+    o0 = (torch.randn(B, H, Lq, d, generator=g) * 0.5).to(torch.bfloat16)
+    out = ops.csp_attn(qg, kg, vg, scale, tidx.cuda(), tcnt.cuda(), o0.cuda(), -1)
+    assert close(out, oracle.csp_attn(q, k, v, scale, tidx, tcnt, o0, -1)), (B, H, Lq, Lk, "csp")
+
+
 def test_token_lists_slice_matches_full_launch():
     """A (batch, head) slice launched alone must reproduce a launch of 512 groups (two workgroups per CU on
     a 256-CU part) bit for bit: the result of a group does not depend on how many others share the launch,
@@ -131,9 +164,10 @@ def _csp_abi(q, k, v, idx, cnt, o0, group_rows, o_scale):
     return st, out
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [64, 128, 256])
 def test_token_lists_every_workgroup_shape(d):
-    """Query groups of 192 rows run as 8-wave workgroups (six computing waves + two fetch waves), other multiples
+    """Query groups of 192 rows run as 8-wave workgroups (six computing waves + two fetch waves; at head_dim 256 as
+    two 3-wave workgroups), other multiples
     of 96 / 64 rows as 3- / 2-wave workgroups that fetch for themselves.  Each variant against the oracle at its
     own group size, and, with every 192-row list repeated for its 96- / 64-row parts, bit for bit against each
     other: the arithmetic of a query row does not depend on the workgroup shape."""
