@@ -455,3 +455,39 @@ def test_head_dim_256():
     kq, vq = k[:, :1].contiguous(), v[:, :1].contiguous()
     og, _ = ops.dense_attn(qg, kq.cuda(), vq.cuda())
     check_o(og, oracle.dense_attn(q, kq.expand(-1, H, -1, -1), vq.expand(-1, H, -1, -1))[0], "gqa d=256")
+
+
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_memory_behind_the_last_key_never_reaches_the_result(d):
+    """K and V are views whose storage continues with NaN rows behind the last key (and NaN heads around them): a
+    ragged last tile, the unused sub-tiles of a 256-key block and the two-tile prefetch must not let them into ``o``
+    (a masked probability is an exact zero, and 0 * NaN would still be NaN)."""
+    from lvar_amd import mask_build as mb, sparse_attn_ops as ops
+    B, H, Lq, Lk, pad = 1, 3, 200, 333, 400
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=5)
+
+    def poisoned(t):
+        big = torch.full((B, H, Lk + pad, d), float("nan"), dtype=torch.bfloat16, device="cuda")
+        big[:, :, :Lk] = t.cuda()
+        return big[:, :, :Lk]
+
+    qg, kg, vg = q.cuda(), poisoned(k), poisoned(v)
+    assert not kg.is_contiguous()
+    o_ref, M_ref, L_ref = oracle.dense_attn(q, k, v)
+    o, (M, L) = ops.dense_attn(qg, kg, vg)
+    check_o(o, o_ref, "dense")
+    check_lse(M, L, M_ref, L_ref)
+    o2, cs, _ = ops.dense_colsum_attn(qg, kg, vg)
+    _, cs_ref, _ = oracle.dense_colsum_attn(q, k, v)
+    check_o(o2, o_ref, "dense + colsum")
+    assert torch.allclose(cs.cpu(), cs_ref, rtol=1e-3, atol=1e-6)
+    for bq, bk in [(128, 64), (64, 64), (128, 128), (128, 256), (64, 256)]:
+        nq, nk = (Lq + bq - 1) // bq, (Lk + bk - 1) // bk
+        mask = torch.rand(B, H, nq, nk, generator=torch.Generator().manual_seed(bq + bk)) < 0.5
+        mask[..., -1] = True     # the ragged last key block is always attended
+        num, idx = oracle.block_mask_to_lists(mask)
+        ob, _ = ops.block_sparse_attn(qg, kg, vg, num.cuda(), idx.cuda(), bq, bk)
+        check_o(ob, oracle.block_sparse_attn(q, k, v, num, idx, bq, bk)[0], f"block {bq}x{bk}")
+    inds, counts = mb.topk_index_list(cs, 0.3)
+    out = ops.csp_attn(qg, kg, vg, None, inds, counts, o, -1)
+    check_o(out, oracle.csp_attn(q, k, v, None, inds.cpu(), counts.cpu(), o.cpu(), -1), "token lists")
