@@ -61,7 +61,7 @@ typedef struct {
 } lvar_workspace_t;
 
 /* Bytes of a workspace that lets every balanced launch of the current device use all its slots
- * (head_dim 64 or 128; head_dim 256 has no balanced launch: LVAR_EUNSUPPORTED), or a negative LVAR_E* code. */
+ * (head_dim 64 or 128; head_dim 256 has no balanced launch and gets the 4 KiB minimum), or a negative LVAR_E* code. */
 int64_t lvar_attn_workspace_bytes(int head_dim);
 
 /* Workgroups a *_ws_fwd launch of these sizes would run as a balanced launch on the current device, 0 if it

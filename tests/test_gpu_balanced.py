@@ -252,3 +252,18 @@ def test_balanced_share_and_piece_knobs(ops):
             assert counters_zero(ops, qg)
     finally:
         ops.set_balanced_launch(True, 0, 0)
+
+
+def test_head_dim_256_takes_the_plain_launch(ops):
+    """head_dim 256 has no balanced launch: the planning query says 0, the size query returns the 4 KiB minimum and
+    the workspace entry point gives the plain launch's result bit for bit."""
+    from lvar_amd import _lib
+    lib = _lib.load()
+    B, H, Lq, Lk, d = 1, 4, 576, 1497, 256
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=2, amp=0.7)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    assert int(lib.lvar_attn_workspace_bytes(d)) == 4096
+    assert plan(ops, 0, qg, kg) == 0
+    a1, a2, b = both(ops, lambda: ops.dense_attn(qg, kg, vg))
+    assert same(a1, b) and same(a2, b)
+    assert close(b[0], oracle.dense_attn(q, k, v)[0])
