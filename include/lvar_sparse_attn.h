@@ -37,8 +37,8 @@ typedef struct {
 
 /*
  * Partial-result workspace of the balanced launches (the *_ws_fwd entry points): device memory owned by the
- * caller, 256-byte aligned, whose first 4096 bytes must be zero before its first use (the library leaves them zero
- * after every launch).  With it, a launch whose plain grid would fill the chip unevenly (at most 1024 query tiles
+ * caller, 256-byte aligned; its contents need no preparation (a balanced launch clears the arrival counters it is
+ * going to use with a small kernel ahead of the attention kernel, and leaves them zero when it ends).  With it, a launch whose plain grid would fill the chip unevenly (at most 1024 query tiles
  * and fewer than four rounds of workgroups: the middle scales of a next-scale-prediction schedule, few query tiles
  * with long or ragged lists) picks a share of about (all list entries) / (resident workgroup slots), cuts every
  * query tile whose list is long enough into round(entries / share) pieces of equal length and runs one workgroup
@@ -64,8 +64,10 @@ typedef struct {
  * (head_dim 64 or 128; head_dim 256 has no balanced launch and gets the 4 KiB minimum), or a negative LVAR_E* code. */
 int64_t lvar_attn_workspace_bytes(int head_dim);
 
-/* Workgroups a *_ws_fwd launch of these sizes would run as a balanced launch on the current device, 0 if it
- * would run as the plain launch; kind 0 = dense, 1 = block list (block_k 64, 128 or 256, list_len = nk_max; group_rows is only looked at for the value 64: query blocks of 64 rows always run as the plain launch),
+/* Shares (resident workgroup slots) that a *_ws_fwd launch of these sizes is planned for as a balanced launch on the
+ * current device, 0 if it would run as the plain launch.  For dense attention (kind 0) the answer is the launch's own
+ * decision; for tile lists (kinds 1 and 2) it is an upper bound: the kernel looks at the real list lengths and leaves
+ * every query tile whole (the plain launch's work split) when no list is long enough to cut.  kind 0 = dense, 1 = block list (block_k 64, 128 or 256, list_len = nk_max; group_rows is only looked at for the value 64: query blocks of 64 rows always run as the plain launch),
  * 2 = token list (group_rows, list_len = idx_row_stride).  Pure planning: nothing is launched. */
 int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, int H, int Lq, int Lk, int list_len,
                                   int head_dim, lvar_workspace_t workspace);

@@ -29,15 +29,8 @@
 
 namespace lvar {
 
-int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub, int64_t ws_bytes, int& min_share, int& min_piece);
-int64_t sk_plan_bytes(int P);
-
-#ifndef LVAR_AHEAD
-#define LVAR_AHEAD 4
-#endif
-#ifndef LVAR_EXP_IN_A
-#define LVAR_EXP_IN_A 24   // of the 32 exp2 per lane and tile, how many run next to the QK MFMAs
-#endif
+constexpr int READ_AHEAD = 4;    // operand fragments requested from LDS this many MFMAs before their use
+constexpr int EXP_IN_QK = 24;    // of the 32 exp2 per lane and tile, how many run next to the QK MFMAs
 
 // First S element of softmax slot g: EA elements spread over the NQK steps of the QK phase, the other
 // 32 - EA over the first HB steps of the PV phase; slots before 0 and after the last one are empty.
@@ -469,7 +462,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       // compiler from regrouping it.  Phase A: QK MFMA j | K-fragment read j+4 | softmax slot j of
       // S(t).  Phase B: PV MFMA j | the two transposing V reads of MFMA j+4 | the last softmax slots
       // of S(t) (first half) or a slice of the row-maximum reduction of S(t+1) (second half).
-      constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = LVAR_AHEAD;
+      constexpr int NQK = 2 * KS, NPV = LSE_ONLY ? 0 : 4 * MTD, AHEAD = READ_AHEAD;
       const char* kbuf = smem + (1 - PAR) * TILE;
       const char* vbuf = smem + (2 + PAR) * TILE;
       auto kread = [&](int j) -> bf16x8 {
@@ -512,7 +505,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
           la += r;
         }
       };
-      using Sch = ExpSlots<2 * KS, (LSE_ONLY ? 0 : 4 * MTD) / 2, LSE_ONLY ? 32 : LVAR_EXP_IN_A>;
+      using Sch = ExpSlots<2 * KS, (LSE_ONLY ? 0 : 4 * MTD) / 2, LSE_ONLY ? 32 : EXP_IN_QK>;
       auto softmax_step = [&](auto gc) {
         constexpr int g = decltype(gc)::value;
         static_for<Sch::lo(g - 2), Sch::lo(g - 1)>(st_sum);
@@ -866,7 +859,14 @@ __global__ __launch_bounds__(NWAVES * 64, (NWAVES <= 4 ? 2 : 1)) void attn_fwd_b
 #endif
 }
 
-// Item table of a balanced launch over tile lists, from the list lengths: one workgroup.
+// words [0, n) of a device buffer := 0 (a kernel, not hipMemsetAsync: callers may be capturing a HIP graph)
+__global__ void zero_words_kernel(uint32_t* dst, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = 0u;
+}
+
+// Item table of a balanced launch over tile lists, from the list lengths: one workgroup.  Also clears the arrival
+// counters of the launch's query tiles, so that a launch does not depend on what the last one left in the workspace.
 template <int WGROWS, int MODE>
 __global__ __launch_bounds__(256) void plan_kernel(const AttnParams p, int* plan) {
   __shared__ int units[SK_MAX_QTILES];    // units of tile u
@@ -881,6 +881,7 @@ __global__ __launch_bounds__(256) void plan_kernel(const AttnParams p, int* plan
     const int g = (qt * WGROWS) / p.group_rows;
     const int cnt = max(0, min(p.cnt[b * p.cnt_sb + h * p.cnt_sh + g], p.list_len));
     units[u] = (MODE == MODE_BLOCK) ? cnt : ((cnt + 63) >> 6);
+    p.sk_counters[u] = 0;
   }
   __syncthreads();
   if (wave == 0) {
@@ -966,15 +967,18 @@ static int launch_one(const AttnParams& p0, hipStream_t stream) {
     p.sk_uniform_n = 0;
     if (p.sk_wgs > 0 && dense) {
       // all lists have (Lk + 63) / 64 entries: the pieces per tile follow from the sizes alone
-      const int T = (int)per_tile, U = p.total_wg * T;
-      const int S = sk_share(U, p.sk_wgs, p.sk_min_share);
-      const int n = sk_worth_cutting(U, S, p.total_wg, p.sk_wgs) ? sk_pieces(T, S, p.sk_min_piece) : 1;
-      if (n > 1 && (int64_t)n * p.total_wg <= 2 * p.sk_wgs) p.sk_uniform_n = n; else p.sk_wgs = 0;   // whole tiles: the plain launch
+      p.sk_uniform_n = sk_dense_pieces(p.total_wg, (int)per_tile, p.sk_wgs, p.sk_min_share, p.sk_min_piece);
+      if (p.sk_uniform_n == 0) p.sk_wgs = 0;   // whole tiles: the plain launch
     }
     if constexpr (NWAVES != 2 && D <= 128) if (p.sk_wgs > 0) {
       p.sk_counters = (int*)p.sk_ws;
       p.sk_slots = (float*)((char*)p.sk_ws + SK_COUNTER_BYTES + sk_plan_bytes(p.sk_wgs));
       int grid_sk;
+      if (p.sk_uniform_n > 0 || p.sk_plan) {
+        // no table kernel ahead of this launch: the arrival counters are cleared by a fill of their own
+        hipLaunchKernelGGL(zero_words_kernel, dim3((p.total_wg + 255) / 256), dim3(256), 0, stream, (uint32_t*)p.sk_counters, p.total_wg);
+        if (hipGetLastError() != hipSuccess) return LVAR_ELAUNCH;
+      }
       if (p.sk_uniform_n > 0) {
         grid_sk = ((p.total_wg * p.sk_uniform_n + 7) / 8) * 8;
       } else {
@@ -1059,6 +1063,16 @@ int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub
   if (P == 0) return 0;
   if (total_wg < slots && 2 * per_tile < 3 * (int64_t)min_share) return 0;
   return P;
+}
+
+// Pieces per query tile of a balanced dense launch (every list has T tiles) on sk_wgs shares, or 0 when the tiles
+// stay whole or the pieces would not fit the launch's slots: then the launch is the plain one.
+int sk_dense_pieces(int total_wg, int T, int sk_wgs, int min_share, int min_piece) {
+  if (sk_wgs <= 0 || total_wg <= 0 || T <= 0) return 0;
+  const int U = total_wg * T;
+  const int S = sk_share(U, sk_wgs, min_share);
+  const int n = sk_worth_cutting(U, S, total_wg, sk_wgs) ? sk_pieces(T, S, min_piece) : 1;
+  return (n > 1 && (int64_t)n * total_wg <= 2 * (int64_t)sk_wgs) ? n : 0;
 }
 
 // bytes of the item-table area of a workspace for P shares (256-byte granules)

@@ -15,12 +15,6 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace {
 
-// words [0, n) of a device buffer := 0 (a kernel, not hipMemsetAsync: callers may be capturing a HIP graph)
-__global__ void zero_words_kernel(uint32_t* dst, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) dst[i] = 0u;
-}
-
 // Device address of this GPU's copy of `scratch`, looked up once per device with that device current.
 void* static_scratch() {
   static std::atomic<void*> ptrs[64];
@@ -225,16 +219,26 @@ int lvar_csp_attn_upsample_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_
                     B, H, Lq, Lk, head_dim, o_scale, scale, &workspace, stream);
 }
 
-static int block_sparse_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
-                               const int32_t* kv_num_blocks, int64_t stride_nb_b, int64_t stride_nb_h,
-                               const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
-                               int64_t stride_ki_q, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
-                               int head_dim, float scale, const lvar_workspace_t* ws, void* stream) {
+// argument checks of the block-list entry points (everything but the workspace)
+static int block_sparse_check(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, const int32_t* kv_num_blocks,
+                              const int32_t* kv_indices, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
+                              int head_dim, float scale) {
   if (!shape_ok(B, H, Lq, Lk, scale) || !view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o)) return LVAR_EINVAL;
   if (!kv_span_ok(k, Lk, head_dim) || !kv_span_ok(v, Lk, head_dim)) return LVAR_EINVAL;
   if (!kv_num_blocks || !kv_indices || nk_max <= 0 || o.stride_row <= 0) return LVAR_EINVAL;
   // query blocks of 64 rows (two-wave workgroups) or a multiple of 128 rows (128-row workgroups that share a list)
   if ((block_q != 64 && (block_q <= 0 || block_q % 128 != 0)) || (block_k != 64 && block_k != 128 && block_k != 256)) return LVAR_EUNSUPPORTED;
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256) return LVAR_EUNSUPPORTED;
+  return LVAR_OK;
+}
+
+static int block_sparse_common(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
+                               const int32_t* kv_num_blocks, int64_t stride_nb_b, int64_t stride_nb_h,
+                               const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
+                               int64_t stride_ki_q, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
+                               int head_dim, float scale, const lvar_workspace_t* ws, void* stream) {
+  const int chk = block_sparse_check(q, k, v, o, kv_num_blocks, kv_indices, nk_max, block_q, block_k, B, H, Lq, Lk, head_dim, scale);
+  if (chk != LVAR_OK) return chk;
   AttnParams p{};
   fill_qkv(p, q, k, v);
   p.o = (bf16_t*)o.ptr; p.o_sb = o.stride_b; p.o_sh = o.stride_h; p.o_sr = o.stride_row;
@@ -290,7 +294,10 @@ int lvar_attn_balanced_workgroups(int kind, int group_rows, int block_k, int B, 
   const int64_t tiles = (int64_t)B * H * ((Lq + rows - 1) / rows);
   if (tiles > 0x7fffffff) return 0;
   int share = workspace.min_share_tiles, piece = workspace.min_piece_tiles;
-  return sk_plan((int)tiles, nwaves, sk_slot_floats(head_dim, mode, nwaves), per_tile, sub, workspace.bytes, share, piece);
+  const int P = sk_plan((int)tiles, nwaves, sk_slot_floats(head_dim, mode, nwaves), per_tile, sub, workspace.bytes, share, piece);
+  // dense attention: the launch code takes the plain launch when the tiles stay whole (the same decision, shared)
+  if (kind == 0 && P > 0 && sk_dense_pieces((int)tiles, (int)per_tile, P, share, piece) == 0) return 0;
+  return P;
 }
 
 int lvar_block_sparse_attn_static_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_t v, lvar_tensor_t o, float* M, float* L,
@@ -298,18 +305,17 @@ int lvar_block_sparse_attn_static_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_ten
                                       const int32_t* kv_indices, int64_t stride_ki_b, int64_t stride_ki_h,
                                       int64_t stride_ki_q, int nk_max, int block_q, int block_k, int B, int H, int Lq, int Lk,
                                       int head_dim, float scale, void* stream) {
-  if (B <= 0 || H <= 0 || Lq <= 0) return LVAR_EINVAL;
+  // arguments first: a call that is refused must not have touched the scratch that a launch in flight may be using
+  const int st = block_sparse_check(q, k, v, o, kv_num_blocks, kv_indices, nk_max, block_q, block_k, B, H, Lq, Lk, head_dim, scale);
+  if (st != LVAR_OK) return st;
   // the scratch holds the counters and the item table of at most LVAR_STATIC_MAX_QUERY_TILES query tiles
   const int wg_rows = block_q == 64 ? 64 : 128;
   const int64_t tiles = (int64_t)B * H * ((Lq + wg_rows - 1) / wg_rows);
   if (tiles > LVAR_STATIC_MAX_QUERY_TILES || head_dim > 128) return LVAR_ETOOBIG;
   void* ptr = static_scratch();
   if (!ptr) return LVAR_ELAUNCH;
-  // The array keeps what the last call left: the arrival counters must start at zero (they do after a launch that
-  // ran to its end; a fill makes that independent of the past).
-  hipLaunchKernelGGL(zero_words_kernel, dim3((int)(SK_COUNTER_BYTES / 4 / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (uint32_t*)ptr, (int)(SK_COUNTER_BYTES / 4));
-  if (hipGetLastError() != hipSuccess) return LVAR_ELAUNCH;
+  // The array keeps what the last call left; a balanced launch clears the arrival counters it is going to use
+  // itself (table kernel or fill kernel ahead of the attention kernel), a plain launch never touches the array.
   lvar_workspace_t ws{};
   ws.ptr = ptr;
   ws.bytes = kStaticScratchBytes;

@@ -130,6 +130,7 @@ int launch_attn(const AttnParams& p, int head_dim, int mode, bool accum, bool ls
 int launch_colsum(const ColsumParams& p, int head_dim, hipStream_t s);
 int sk_slot_floats(int head_dim, int mode, int nwaves);
 int sk_plan(int total_wg, int nwaves, int slot_floats, int64_t per_tile, int sub, int64_t ws_bytes, int& min_share, int& min_piece);
+int sk_dense_pieces(int total_wg, int T, int sk_wgs, int min_share, int min_piece);   // dense attention: pieces per query tile, 0 = plain launch
 int device_cus();   // compute units of the current device (cached), 0 on error
 constexpr int64_t SK_COUNTER_BYTES = 4096;   // head of the workspace: one int32 arrival counter per query tile
 int64_t sk_plan_bytes(int P);                // then the item table, then 2 * P slots

@@ -20,7 +20,7 @@ INFINITY_SCALES = (1, 2, 4, 6, 8, 12, 16, 20, 24, 32, 40, 48, 64)
 __all__ = [
     "INFINITY_SCALES", "scale_offsets", "indices_count", "topk_index_list", "map_inds_counts_across_scales",
     "local_group_runs", "append_local_run", "upsample_ocache", "flex_block_mask", "block_mask_to_lists",
-    "key_block_sums", "topk_block_lists", "sink_window_base_mask", "sink_window_topk_block_mask",
+    "key_block_sums", "topk_block_lists", "block_keep_count", "sink_window_base_mask", "sink_window_topk_block_mask",
     "video_window_base_mask", "video_window_topk_block_lists",
 ]
 
@@ -48,8 +48,8 @@ def topk_index_list(bs: torch.Tensor, top_keys: float, multiple_of: Optional[int
     int32 [B,H,G].  Padding columns are zero-filled unless ``zero_tail`` is false (the reference leaves them
     uninitialised, sparse_attn.py:1031-1034; they are never read).  ``order="value"`` lists the keys by descending score as ``torch.topk`` does,
     ``order="index"`` by ascending key (same set; the attention kernels do not depend on the order
-    and gather ascending lists faster).  A tensor on a HIP device goes through the radix-select
-    kernel (:func:`lvar_amd.sparse_attn_ops.topk_token_lists`, ties to the smaller key)."""
+    and gather ascending lists faster).  The selection is the radix-select kernel
+    (:func:`lvar_amd.sparse_attn_ops.topk_token_lists`, ties to the smaller key): ``bs`` must live on a HIP device."""
     cfg = get_kernel_config_attn()
     m = cfg["counts_multiple_of"] if multiple_of is None else multiple_of
     B, H, G, Lk = bs.shape
@@ -58,15 +58,8 @@ def topk_index_list(bs: torch.Tensor, top_keys: float, multiple_of: Optional[int
         raise ValueError(f"top-k count {cnt} exceeds key length {Lk}")
     if order not in ("value", "index"):
         raise ValueError("order must be 'value' or 'index'")
-    if bs.is_cuda:
-        from . import sparse_attn_ops as ops
-        return ops.topk_token_lists(bs, cnt, out_len=Lk, order=order, zero_tail=zero_tail)
-    inds = torch.zeros((B, H, G, Lk), dtype=torch.int32, device=bs.device)
-    if cnt > 0:
-        top = torch.topk(bs, k=cnt, dim=-1).indices
-        inds[..., :cnt] = (top if order == "value" else top.sort(-1).values).to(torch.int32)
-    counts = torch.full((B, H, G), cnt, dtype=torch.int32, device=bs.device)
-    return inds, counts
+    from . import sparse_attn_ops as ops
+    return ops.topk_token_lists(bs, cnt, out_len=Lk, order=order, zero_tail=zero_tail)   # HIP tensors only
 
 
 def map_inds_counts_across_scales(inds_S: torch.Tensor, counts_S, cur_q_len: int, cur_k_len: int,
@@ -194,18 +187,10 @@ def flex_block_mask(q_scale_idx: int, kernel_schedule: Sequence[int], attn_sink_
 
 def block_mask_to_lists(mask: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """bool [..., nQ, nK] -> flex ``BlockMask`` lists: ``kv_num_blocks`` int32 [..., nQ] and
-    ``kv_indices`` int32 [..., nQ, nK] (kept blocks first, ascending; unused tail zero).  A mask on
-    a HIP device is compacted by one kernel (:func:`lvar_amd.sparse_attn_ops.mask_to_lists`)."""
-    if mask.is_cuda:
-        from . import sparse_attn_ops as ops
-        return ops.mask_to_lists(mask, 1)
-    nK = mask.shape[-1]
-    num = mask.sum(-1, dtype=torch.int32)
-    # kept blocks sort before dropped ones, both in ascending block order
-    key = (~mask).to(torch.int32) * nK + torch.arange(nK, device=mask.device, dtype=torch.int32)
-    order = torch.argsort(key, dim=-1).to(torch.int32)
-    keep = torch.arange(nK, device=mask.device) < num.unsqueeze(-1)
-    return num, torch.where(keep, order, torch.zeros_like(order)).contiguous()
+    ``kv_indices`` int32 [..., nQ, nK] (kept blocks first, ascending; unused tail zero): one compaction
+    kernel (:func:`lvar_amd.sparse_attn_ops.mask_to_lists`); the mask must live on a HIP device."""
+    from . import sparse_attn_ops as ops
+    return ops.mask_to_lists(mask, 1)
 
 
 def key_block_sums(cs: torch.Tensor, block_k: int = 64) -> torch.Tensor:
@@ -220,16 +205,22 @@ def topk_block_lists(block_scores: torch.Tensor, keep_ratio: float, k_len: Optio
     """Best-scoring key blocks per row as ascending block lists.  The number kept follows the
     reference's token-count formula when ``k_len`` is given, ``block_k*round(keep_ratio*k_len/block_k)``
     tokens = that many blocks (models/sparvar/sparse_attn.py:1012), else ``round(keep_ratio*nK)``;
-    at least one block is kept."""
-    nK = block_scores.shape[-1]
+    at least one block is kept.  ``block_scores`` fp32 ``[B,H,nQ,nK]`` on a HIP device."""
+    k = block_keep_count(keep_ratio, block_scores.shape[-1], k_len, block_k)
+    from . import sparse_attn_ops as ops
+    num, idx = ops.block_topk_lists(block_scores, k)          # HIP selection kernel; ties go to the smaller block
+    return num, idx[..., :k].contiguous()
+
+
+def block_keep_count(keep_ratio: float, n_blocks: int, k_len: Optional[int] = None, block_k: int = 64) -> int:
+    """Key blocks kept per row by :func:`topk_block_lists`: the reference's token count
+    ``block_k*round(keep_ratio*k_len/block_k)`` (models/sparvar/sparse_attn.py:1012) in blocks when ``k_len`` is
+    given, else ``round(keep_ratio*n_blocks)``; at least one, at most all."""
     if k_len is not None:
         k = indices_count(keep_ratio, k_len, block_k) // block_k
     else:
-        k = int(round(keep_ratio * nK))
-    k = max(1, min(nK, k))
-    idx = torch.topk(block_scores, k=k, dim=-1).indices.sort(-1).values.to(torch.int32)
-    num = torch.full(block_scores.shape[:-1], k, dtype=torch.int32, device=block_scores.device)
-    return num, idx.contiguous()
+        k = int(round(keep_ratio * n_blocks))
+    return max(1, min(n_blocks, k))
 
 
 def sink_window_base_mask(block_q: int = 128, block_k: int = 64, sink_scale: int = 7, window: int = 2,

@@ -24,7 +24,7 @@ from .sparse_attn_config import get_kernel_config_attn
 
 __all__ = [
     "dense_attn", "dense_colsum_attn", "dense_colsum_attn_s", "dense_colsum_attn_q", "colsum",
-    "csp_attn", "csp_attn_delta", "block_sparse_attn", "block_topk_lists", "ShapeError", "set_balanced_launch",
+    "csp_attn", "csp_attn_delta", "block_sparse_attn", "block_topk_lists", "mask_to_indices", "topk_indices", "ShapeError",
 ]
 
 
@@ -137,12 +137,12 @@ _balanced = False
 _NO_WORKSPACE = _lib.LvarWorkspace(None, 0, 0, 0)
 
 
-def set_balanced_launch(enabled: bool, min_share_tiles: int = 0, min_piece_tiles: int = 0) -> None:
-    """Switches the balanced launches on or off (default off): with them, an attention call whose plain grid would
-    fill the chip unevenly (few query tiles with long or ragged lists) cuts long tile lists into pieces of about
-    one share of the whole launch, runs one workgroup per piece and adds the pieces up in a partial-result
-    workspace.  On a 256-CU part the measured gain at the Infinity-2B shapes is within +-10 % of the plain launch
-    (a compute unit already walks ~1 key tile per microsecond however the tiles are dealt), hence opt-in.
+def _set_balanced_launch(enabled: bool, min_share_tiles: int = 0, min_piece_tiles: int = 0) -> None:
+    """Test and measurement hook, not part of the operator API: routes the attention operators through the
+    ``*_ws_fwd`` entry points with a workspace, so that launches whose plain grid would fill the chip unevenly are cut
+    into pieces (the balanced launch of the C ABI).  The operators themselves always take the plain launch: on a
+    256-CU part the balanced one measures within +-10 % of it at the Infinity-2B shapes and mostly slower.  Callers
+    that want it (few query tiles with very long lists) call the ``*_ws_fwd`` entry points with their own workspace.
     ``min_share_tiles`` / ``min_piece_tiles`` override the library defaults (0 = default)."""
     global _balanced
     _balanced = bool(enabled)
@@ -192,7 +192,7 @@ def _dense_launch(q, k, v, scale, want_o=True, want_ml=True, want_lse2=False):
 def dense_attn(q, k, v, scale=None):
     """Dense flash attention, ``(o, (M, L))`` (reference ``dense_attn``, sparse_attn_ops.py:21-59,
     Triton-provider return convention: ``lse`` is the tuple ``(M, L)``, each ``[B,H,Lq,1]``)."""
-    fast = _lib.torch_binding()
+    fast = None if _balanced else _lib.torch_binding()   # (the compiled path takes no workspace)
     if fast is not None:
         # None unless the inputs are the plain contiguous bf16 case
         r = fast.fast_dense_attn(q, k, v, None if scale is None else float(scale)) if isinstance(q, torch.Tensor) else None
@@ -529,6 +529,75 @@ def mask_to_lists(mask, multiple_of: int = 1):
                                            int(multiple_of), _stream(m))
     _lib.check(st, "lvar_mask_to_lists")
     return cnt, idx
+
+
+def mask_to_indices(mask, multiple_of: int, pad_to_multiple_of: int = 192):
+    """``[indices, counts]`` of a boolean mask ``[b,h,m,n]`` (reference ``mask_to_indices``, sparse_attn_ops.py:402-407,
+    kernels/chipmunk/csrc/indexed_io/mask_to_indices.cu:96-141): ``indices`` int32 ``[b,h,m,pad_n]`` with ``pad_n`` =
+    ``n`` rounded up to ``pad_to_multiple_of``, ``counts`` int32 ``[b,h,m]`` = the number of set columns rounded up to
+    ``multiple_of``, the padding entries being the lowest unset columns.  The set columns come in ascending order
+    (the reference's order is thread-strided) and the padded count is capped at ``n``; columns from the count on are
+    zero up to ``n`` and left as allocated beyond (the reference leaves all of them as allocated)."""
+    _require(mask.dim() == 4, "mask must be 4-dimensional [b, h, m, n]")
+    if mask.dtype != torch.bool:
+        raise TypeError("mask must be bool type")
+    if not mask.is_cuda:
+        raise RuntimeError("mask must live on a HIP device; lvar_amd has no CPU path")
+    _require(multiple_of >= 1 and pad_to_multiple_of >= 1, "multiple_of and pad_to_multiple_of must be positive")
+    m = mask.contiguous().view(torch.uint8)
+    b, h, rows_m, n = m.shape
+    pad_n = (n + pad_to_multiple_of - 1) // pad_to_multiple_of * pad_to_multiple_of
+    idx = torch.empty((b, h, rows_m, pad_n), dtype=torch.int32, device=m.device)
+    cnt = torch.empty((b, h, rows_m), dtype=torch.int32, device=m.device)
+    if n > 0 and cnt.numel() > 0:
+        with _on_device(m):
+            st = _lib.load().lvar_mask_to_lists(m.data_ptr(), n, idx.data_ptr(), pad_n, cnt.data_ptr(), b * h * rows_m, n,
+                                               int(multiple_of), _stream(m))
+        _lib.check(st, "lvar_mask_to_lists")
+    return [idx, cnt]
+
+
+def topk_indices(activations, indices_out, counts_out, sparsity_amount: float, multiple_of: int, rk: float = 0.0) -> None:
+    """In-place counterpart of the reference's ``topk_indices`` (sparse_attn_ops.py:381-389,
+    kernels/chipmunk/csrc/indexed_io/topk_indices.cu:26-175): for every row of ``activations`` ``[batch, rows, cols]``
+    keep the columns at or above the ``sparsity_amount`` quantile, plus each other column with probability ``rk``,
+    pad the count to a multiple of ``multiple_of`` with the lowest unselected columns, and write the list into
+    ``indices_out`` int32 ``[batch, rows, cols]`` (entries beyond the count are left as the caller filled them) and the
+    count into ``counts_out`` int32 ``[batch, rows]``.  ``sparsity_amount`` 0 keeps every column, 1 none.
+    The reference estimates the quantile from the first 1024 entries of a row with a block sort; here it is exact over
+    the whole row (radix select: the ``cols - int(cols * sparsity_amount)`` largest entries, ties to the smaller
+    column), and the list is in ascending column order."""
+    _require(activations.dim() == 3, "activation must be 3-dimensional [batch, rows, cols]")
+    _require(indices_out.dim() == 3 and tuple(indices_out.shape) == tuple(activations.shape),
+             "indices must be 3-dimensional [batch, rows, cols]")
+    _require(counts_out.dim() == 2 and tuple(counts_out.shape) == tuple(activations.shape[:2]),
+             "counts must be 2-dimensional [batch, rows]")
+    _require(0.0 <= sparsity_amount <= 1.0, "sparsity_amount must be between 0 and 1")
+    _require(multiple_of >= 1, "multiple_of must be positive")
+    if not activations.is_cuda:
+        raise RuntimeError("activation must live on a HIP device; lvar_amd has no CPU path")
+    if indices_out.dtype != torch.int32 or counts_out.dtype != torch.int32 or not indices_out.is_contiguous() \
+            or not counts_out.is_contiguous():
+        raise TypeError("indices and counts must be contiguous int32 tensors")
+    batch, rows, cols = activations.shape
+    if sparsity_amount == 1.0:
+        indices_out.fill_(-1)
+        counts_out.zero_()
+        return
+    keep = cols - int(cols * float(sparsity_amount))
+    sel, _ = topk_token_lists(activations, keep, out_len=cols, zero_tail=False)
+    if rk <= 0.0 and keep % multiple_of == 0:
+        indices_out[..., :keep] = sel[..., :keep]
+        counts_out.fill_(keep)
+        return
+    mask = torch.zeros((1, batch, rows, cols), dtype=torch.bool, device=activations.device)
+    mask[0].scatter_(-1, sel[..., :keep].long(), True)
+    if rk > 0.0:
+        mask |= torch.rand(mask.shape, device=mask.device) < float(rk)
+    idx, cnt = mask_to_indices(mask, multiple_of, 1)
+    width = torch.arange(cols, device=mask.device) < cnt[0].unsqueeze(-1)
+    indices_out.copy_(torch.where(width, idx[0], indices_out))
+    counts_out.copy_(cnt[0])
 
 
 def window_key_scores(q, k, window_keys, kernel_size: int = 5, pooling: str = "avgpool", scale=None):

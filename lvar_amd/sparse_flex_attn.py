@@ -17,8 +17,11 @@ class SparseFlexAttn(torch.nn.Module):
     def __init__(self, scale_schedule: Sequence, kernel_schedule: Sequence[int], q_scale_idx: int, attn_sink_scale: int,
                  block_size: int = _DEFAULT_SPARSE_BLOCK_SIZE, num_heads: int = 16, device=None):
         super().__init__()
-        if block_size != 128:
-            raise ValueError("the HIP block-sparse kernel supports 128-row query blocks (block_size=128)")
+        # square blocks, as flex's BLOCK_SIZE=int gives them (basic_sparvar.py:55-72): the sizes the kernel walks
+        if block_size not in (64, 128, 256):
+            raise ValueError("block_size must be 64, 128 or 256 (the block shapes of the HIP block-sparse kernel)")
+        if device is None:
+            device = "cuda"     # the reference builds its mask on 'cuda' too (basic_sparvar.py:70); there is no CPU path
         self.block_size = block_size
         self.num_heads = num_heads
         hw = mb._hw(scale_schedule)

@@ -1,5 +1,5 @@
-"""Torch-library registration of the three attention ops with the schemas the reference registers as
-``torch.ops.chipmunk.*`` (kernels/chipmunk/csrc/chipmunk.cu:57-59), for callers that use the
+"""Torch-library registration of the three attention ops and the two list-building ops with the schemas the reference
+registers as ``torch.ops.chipmunk.*`` (kernels/chipmunk/csrc/chipmunk.cu:57-59, 66-68), for callers that use the
 torch-library entry points directly (``SelfAttention.forward`` calls ``torch.ops.chipmunk.dense_attn``,
 models/sparvar/basic_sparvar.py:384).  Like the reference's CUDA ops the softmax scale is fixed to 1
 (Infinity's cosine attention, dense_attn.cu:161-163); ``lse`` / ``p`` / ``l`` are the reference's
@@ -9,6 +9,8 @@ per-row constant ``1 / (2^M * L)`` with the 1 = e^0 scale folded in, shape ``[B,
     o, lse = torch.ops.lvar.dense_attn(q, k, v)
     o, cs, l = torch.ops.lvar.dense_colsum_attn(q, k, v, lse)
     torch.ops.lvar.csp_attn(q, k, v, o, indices, counts, -1)      # in place on o
+    indices, counts = torch.ops.lvar.mask_to_indices(mask, 64, 192)
+    torch.ops.lvar.topk_indices(activation, indices, counts, 0.8, 64, 0.0)   # in place on indices / counts
 
     lvar_amd.torch_ops.register_as("chipmunk")    # opt-in: the reference's call sites then run unedited
 
@@ -30,6 +32,9 @@ _SCHEMAS = {
     "csp_attn": "csp_attn(Tensor q, Tensor k, Tensor v, Tensor(a!) o, Tensor indices, Tensor indices_counts, int o_scale) -> ()",
     "dense_attn": "dense_attn(Tensor q, Tensor k, Tensor v) -> Tensor[]",
     "dense_colsum_attn": "dense_colsum_attn(Tensor q, Tensor k, Tensor v, Tensor p) -> Tensor[]",
+    # indexed IO (chipmunk.cu:66-68)
+    "topk_indices": "topk_indices(Tensor activation, Tensor(indices!) indices, Tensor counts, float sparsity_amount, int multiple_of, float random_amount) -> ()",
+    "mask_to_indices": "mask_to_indices(Tensor mask, int multiple_of, int pad_to_multiple_of) -> Tensor[]",
 }
 _registered = {}      # namespace -> the torch.library.Library objects that keep the registration alive
 
@@ -70,11 +75,20 @@ def _csp_attn(q, k, v, o, indices, indices_counts, o_scale):
     ops._csp_launch(q, k, v, indices, indices_counts, o, o_scale, 1.0, False, out=o)
 
 
-_IMPLS = {"dense_attn": _dense_attn, "dense_colsum_attn": _dense_colsum_attn, "csp_attn": _csp_attn}
+def _topk_indices(activation, indices, counts, sparsity_amount, multiple_of, random_amount):
+    ops.topk_indices(activation, indices, counts, sparsity_amount, multiple_of, random_amount)
+
+
+def _mask_to_indices(mask, multiple_of, pad_to_multiple_of):
+    return ops.mask_to_indices(mask, multiple_of, pad_to_multiple_of)
+
+
+_IMPLS = {"dense_attn": _dense_attn, "dense_colsum_attn": _dense_colsum_attn, "csp_attn": _csp_attn,
+          "topk_indices": _topk_indices, "mask_to_indices": _mask_to_indices}
 
 
 def register_as(namespace: str) -> None:
-    """Registers the three ops under ``torch.ops.<namespace>`` (idempotent).  ``register_as("chipmunk")`` makes
+    """Registers the ops under ``torch.ops.<namespace>`` (idempotent).  ``register_as("chipmunk")`` makes
     the reference's call sites (``torch.ops.chipmunk.dense_attn`` at basic_sparvar.py:384, the ``cuda`` provider
     branches of sparse_attn_ops.py:55,84,96,289) resolve to this library; it refuses to do so when another
     extension has already registered one of these ops under that name."""

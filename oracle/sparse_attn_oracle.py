@@ -27,7 +27,7 @@ __all__ = [
     "block_sparse_attn", "block_mask_to_lists", "lists_to_block_mask",
     "map_inds_counts_across_scales", "local_window_indices", "crossscale_self_indices",
     "aggregate_group_indices", "upsample_ocache", "flex_block_mask", "infinity_cum",
-    "INFINITY_SCALES", "config2_block_mask", "attn_flops_blocks", "attn_flops_lists",
+    "INFINITY_SCALES", "config2_block_mask", "attn_flops_blocks",
     "topk_token_set", "append_local_run", "mask_to_lists", "window_key_scores",
     "video_window_block_mask", "base_plus_topk_block_mask", "expand_kv_heads",
 ]
@@ -497,13 +497,6 @@ def attn_flops_blocks(kv_num_blocks, kv_indices, Lq, Lk, d, block_q, block_k):
                 cols = torch.clamp(Lk - js * block_k, max=block_k).clamp(min=0).sum().item()
                 total += rows * cols
     return 4 * d * total
-
-
-def attn_flops_lists(counts, Lq, d, bm=192):
-    """``4*d*sum_g rows_g*counts[b,h,g]`` for token-list attention."""
-    B, H, G = counts.shape
-    rows = torch.tensor([min(bm, Lq - g * bm) for g in range(G)], dtype=torch.int64)
-    return int(4 * d * (counts.long() * rows.view(1, 1, G)).sum().item())
 
 
 def video_window_block_mask(frames=8, height=64, width=64, block=128, frame_radius=1, spatial_radius=1):

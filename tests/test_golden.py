@@ -110,9 +110,8 @@ def test_oracle_and_host_mirrors_reproduce_list_kernel_fixture():
     from lvar_amd import mask_build as mb
     z = load("list_kernels.npz")
     assert torch.equal(oracle.topk_token_set(t(z["scores"]), 128), t(z["topk128"]))
-    # the torch host mirrors (CPU path of lvar_amd.mask_build) give the same lists
-    inds, counts = mb.topk_index_list(t(z["scores"]).unsqueeze(0), 128 / 700, multiple_of=64, order="index")
-    assert int(counts[0, 0, 0]) == 128 and torch.equal(inds[0, ..., :128], t(z["topk128"]))
+    # the torch host arithmetic of lvar_amd.mask_build (remap + local-run append) gives the same lists
+    assert mb.indices_count(128 / 700, t(z["scores"]).shape[-1], 64) == 128
     a, c = mb.map_inds_counts_across_scales(t(z["src"]), 192, 2304, 900)
     out, cnt = mb.append_local_run(a, 192, t(z["local"]), 64, 900, multiple_of=64)
     assert torch.equal(out, t(z["remap_concat"])) and torch.equal(cnt, t(z["remap_counts"]))
@@ -129,6 +128,9 @@ def test_hip_matches_list_kernel_fixture():
     z = load("list_kernels.npz")
     idx, cnt = ops.topk_token_lists(t(z["scores"]).cuda(), 128)
     assert torch.equal(idx[..., :128].cpu(), t(z["topk128"])) and bool((cnt == 128).all())
+    from lvar_amd import mask_build as mb
+    inds, counts = mb.topk_index_list(t(z["scores"]).unsqueeze(0).cuda(), 128 / 700, multiple_of=64, order="index")
+    assert int(counts[0, 0, 0]) == 128 and torch.equal(inds[0, ..., :128].cpu(), t(z["topk128"]))
     out, counts = ops.remap_concat_lists(t(z["src"]).cuda(), 192, 2304, 900, t(z["local"]).cuda())
     assert torch.equal(out.cpu(), t(z["remap_concat"])) and torch.equal(counts.cpu(), t(z["remap_counts"]))
     mc, mi = ops.mask_to_lists(t(z["mask"]).cuda(), 64)

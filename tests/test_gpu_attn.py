@@ -329,14 +329,16 @@ def test_block_topk_lists_bit_exact():
     base = mb.sink_window_base_mask()
     target = round(0.25 * 165)
     num, idx = ops.block_topk_lists(scores.cuda(), target, base)
-    n_ref, i_ref = mb.block_mask_to_lists(mb.sink_window_topk_block_mask(scores))
+    n_ref, i_ref = oracle.block_mask_to_lists(oracle.config2_block_mask(scores))
     assert torch.equal(num.cpu(), n_ref) and torch.equal(idx.cpu(), i_ref)
     assert bool((num == target).all())
     # no base mask, plain top-k; target larger than the row keeps everything; target 0 keeps nothing
     s2 = torch.rand(1, 2, 5, 70, generator=g)
     num, idx = ops.block_topk_lists(s2.cuda(), 7)
-    n_ref, i_ref = mb.topk_block_lists(s2, 0.1)
-    assert int(n_ref[0, 0, 0]) == 7 and torch.equal(num.cpu(), n_ref) and torch.equal(idx.cpu()[..., :7], i_ref)
+    n_ref, i_ref = oracle.block_mask_to_lists(oracle.base_plus_topk_block_mask(s2, torch.zeros(5, 70, dtype=torch.bool), 7))
+    assert int(n_ref[0, 0, 0]) == 7 and torch.equal(num.cpu(), n_ref) and torch.equal(idx.cpu(), i_ref)
+    n_mb, i_mb = mb.topk_block_lists(s2.cuda(), 0.1)          # the policy wrapper: round(0.1 * 70) = 7 blocks
+    assert torch.equal(n_mb.cpu(), n_ref) and torch.equal(i_mb.cpu(), i_ref[..., :7]) and i_mb.dtype == torch.int32
     assert bool((idx.cpu()[..., 7:] == 0).all())
     num, idx = ops.block_topk_lists(s2.cuda(), 500)
     assert bool((num == 70).all()) and torch.equal(idx.cpu()[0, 0, 0], torch.arange(70, dtype=torch.int32))

@@ -25,9 +25,9 @@ def lse_close(M, L, M_ref, L_ref, tol=1e-3):
 @pytest.fixture()
 def ops():
     from lvar_amd import sparse_attn_ops as o
-    o.set_balanced_launch(True)
+    o._set_balanced_launch(True)
     yield o
-    o.set_balanced_launch(False)        # the default
+    o._set_balanced_launch(False)        # the default
 
 
 def plan(ops, kind, q, k, group_rows=192, block_k=64, list_len=0):
@@ -45,12 +45,12 @@ def counters_zero(ops, q):
 
 def both(ops, fn):
     """fn() with the balanced launch on (twice) and off."""
-    ops.set_balanced_launch(True)
+    ops._set_balanced_launch(True)
     a1 = fn()
     a2 = fn()
-    ops.set_balanced_launch(False)
+    ops._set_balanced_launch(False)
     b = fn()
-    ops.set_balanced_launch(True)
+    ops._set_balanced_launch(True)
     return a1, a2, b
 
 
@@ -195,6 +195,60 @@ def test_token_lists_balanced_with_fused_upsample(ops):
     assert close(o1[:1, :2], ref, atol=3e-2)
 
 
+def test_dense_attn_operator_goes_through_the_workspace(ops):
+    """With the hook on, ``dense_attn`` leaves its compiled host path (which takes no workspace) and runs the balanced
+    grid: the partial-result slots behind the counters are written, the counters are zero again afterwards."""
+    B, H, Lq, Lk, d = 1, 3, 300, 5000, 64
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=17, amp=0.7)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    ops.dense_attn(qg, kg, vg)                                        # allocates the workspace of this stream
+    assert plan(ops, 0, qg, kg) > 0
+    ws = ops._workspaces[(qg.device.index, ops._stream(qg))][1]
+    ws.zero_()
+    o, (M, L) = ops.dense_attn(qg, kg, vg)
+    assert bool(ws[4096:].any()) and counters_zero(ops, qg)
+    o_ref, M_ref, L_ref = oracle.dense_attn(q, k, v)
+    assert close(o, o_ref) and lse_close(M, L, M_ref, L_ref)
+    # stale arrival counters (a launch cut short, a workspace used before) are cleared by the launch itself
+    ws[:4096] = 0x5a
+    o2, (M2, L2) = ops.dense_attn(qg, kg, vg)
+    assert torch.equal(o2, o) and torch.equal(M2, M) and torch.equal(L2, L)
+    ops._set_balanced_launch(False)
+    ws.zero_()
+    ops.dense_attn(qg, kg, vg)
+    assert not bool(ws.any())                                         # off: the workspace is not touched
+    ops._set_balanced_launch(True)
+
+
+def test_piece_exchange_gives_the_same_bits_launch_after_launch(ops):
+    """The pieces of a cut query tile travel between compute-unit groups through device-coherent stores and loads
+    ordered by the arrival counter alone; a stale read would be a silent wrong answer.  Many-piece launches (a dense
+    one whose every tile is cut eight times, a token-list one with ragged lists) repeated a few hundred times must
+    reproduce the first result bit for bit; the loop stops at the first launch that does not."""
+    from lvar_amd import _lib
+    q, k, v = make_qkv(1, 3, 300, 5000, 64, seed=23, amp=0.7)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    assert plan(ops, 0, qg, kg) > 0
+    first = ops._dense_launch(qg, kg, vg, None)[:3]
+    assert close(first[0], oracle.dense_attn(q, k, v)[0])
+    for rep in range(300):
+        again = ops._dense_launch(qg, kg, vg, None)[:3]
+        assert same(again, first), f"dense launch {rep} differs from the first"
+    g = torch.Generator().manual_seed(29)
+    B, H, Lq, Lk, d, rows = 2, 8, 1600, 2600, 128, 192
+    q, k, v = make_qkv(B, H, Lq, Lk, d, seed=4, amp=0.5)
+    G = (Lq + rows - 1) // rows
+    idx = torch.randint(0, Lk, (B, H, G, Lk), generator=g, dtype=torch.int32).cuda()
+    cnt = torch.randint(0, Lk + 1, (B, H, G), generator=g, dtype=torch.int32).cuda()
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    o0 = torch.zeros_like(qg)
+    assert plan(ops, 2, qg, kg, group_rows=rows, list_len=Lk) > 0
+    first = ops.csp_attn(qg, kg, vg, None, idx, cnt, o0, 1)
+    for rep in range(200):
+        assert torch.equal(ops.csp_attn(qg, kg, vg, None, idx, cnt, o0, 1), first), f"token-list launch {rep} differs from the first"
+    assert counters_zero(ops, qg)
+
+
 def test_small_workspace_and_plain_fallback(ops):
     """A workspace that holds one slot pair per CU halves the workgroups; one too small for that, a null
     workspace, or too little work for a share per workgroup give the plain launch, bit for bit."""
@@ -209,13 +263,13 @@ def test_small_workspace_and_plain_fallback(ops):
 
     def need(P):      # arrival counters, item table for 1024 query tiles + P shares (256-byte granules), 2 * P slots
         return 4096 + ((8 + 8 * (1024 + P)) * 4 + 255) // 256 * 256 + 2 * P * slot
-    ops.set_balanced_launch(False)
+    ops._set_balanced_launch(False)
     o_plain, M_plain, L_plain, _ = ops._dense_launch(qg, kg, vg, None)
-    ops.set_balanced_launch(True)
+    ops._set_balanced_launch(True)
     o_ref, _, _ = oracle.dense_attn(q, k, v)
     assert full >= need(2 * cus)
     for nbytes, want in ((full, 2 * cus), (need(2 * cus), 2 * cus), (need(cus), cus), (need(cus) - 256, 0), (4096, 0)):
-        buf = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        buf = torch.full((nbytes,), 0x33 if want else 0, dtype=torch.uint8, device="cuda")   # contents need no preparation
         ws = _lib.LvarWorkspace(buf.data_ptr(), nbytes, 0, 0)
         assert lib.lvar_attn_balanced_workgroups(0, 0, 0, B, H, Lq, Lk, 0, d, ws) == want
         o = torch.empty_like(qg)
@@ -226,7 +280,7 @@ def test_small_workspace_and_plain_fallback(ops):
         assert st == 0 and close(o, o_ref)
         if want == 0:
             assert torch.equal(o, o_plain) and torch.equal(M, M_plain) and torch.equal(L, L_plain)
-        assert not bool(buf[:4096].any())
+        assert not bool(buf[:4 * B * H * ((Lq + 127) // 128)].any())      # the arrival counters of this launch's query tiles
     # tiny problem: no share of work per workgroup -> plain
     qs, ks = qg[:, :, :64], kg[:, :, :100]
     assert plan(ops, 0, qs.contiguous(), ks.contiguous()) == 0
@@ -246,12 +300,12 @@ def test_balanced_share_and_piece_knobs(ops):
     o_ref, M_ref, L_ref = oracle.dense_attn(q, k, v)
     try:
         for share, piece in ((1, 1), (2, 1), (8, 4), (16, 16), (64, 3)):
-            ops.set_balanced_launch(True, share, piece)
+            ops._set_balanced_launch(True, share, piece)
             o, M, L, _ = ops._dense_launch(qg, kg, vg, None)
             assert close(o, o_ref) and lse_close(M, L, M_ref, L_ref), (share, piece)
             assert counters_zero(ops, qg)
     finally:
-        ops.set_balanced_launch(True, 0, 0)
+        ops._set_balanced_launch(True, 0, 0)
 
 
 def test_head_dim_256_takes_the_plain_launch(ops):

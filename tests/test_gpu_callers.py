@@ -22,7 +22,7 @@ def test_sparse_flex_attn_matches_oracle():
     ks = [-1, -1, -1, -1, 1, 1, 3, 5, 7]
     mod = SparseFlexAttn([(s, s) for s in SCALES9], ks, q_scale_idx=8, attn_sink_scale=3, num_heads=2)
     mask = oracle.flex_block_mask(8, ks, 3, 128, scales=SCALES9)
-    assert torch.equal(mod.block_level_mask, mask)
+    assert torch.equal(mod.block_level_mask.cpu(), mask)
     q, k, v = make_qkv(2, 2, 576, 1497, 128, seed=8, amp=0.5)
     num, idx = oracle.block_mask_to_lists(mask.expand(2, 2, *mask.shape))
     ref, _, _ = oracle.block_sparse_attn(q, k, v, num, idx, 128, 128, scale=1.0)
@@ -31,6 +31,71 @@ def test_sparse_flex_attn_matches_oracle():
     assert out.dtype == torch.bfloat16 and close(out, ref)
     with pytest.raises(ValueError):
         mod(q[:, :, :100].cuda(), k.cuda(), v.cuda())
+    # the other square block sizes flex takes as BLOCK_SIZE=int (basic_sparvar.py:55-72) and the kernel walks
+    for bs in (64, 256):
+        mod_b = SparseFlexAttn([(s, s) for s in SCALES9], ks, q_scale_idx=8, attn_sink_scale=3, block_size=bs, num_heads=2)
+        mask_b = oracle.flex_block_mask(8, ks, 3, bs, scales=SCALES9)
+        assert torch.equal(mod_b.block_level_mask.cpu(), mask_b)
+        num_b, idx_b = oracle.block_mask_to_lists(mask_b.expand(2, 2, *mask_b.shape))
+        ref_b, _, _ = oracle.block_sparse_attn(q, k, v, num_b, idx_b, bs, bs, scale=1.0)
+        assert close(mod_b(q.float().cuda(), k.float().cuda(), v.cuda(), scale=1.0), ref_b), bs
+    with pytest.raises(ValueError):
+        SparseFlexAttn([(s, s) for s in SCALES9], ks, q_scale_idx=8, attn_sink_scale=3, block_size=96)
+
+
+def test_torch_ops_list_building_schemas():
+    """``torch.ops.chipmunk.mask_to_indices`` / ``topk_indices`` called as the reference's wrappers call them
+    (kernels/sparse_attn/sparse_attn_ops.py:381-407; schemas of kernels/chipmunk/csrc/chipmunk.cu:66-68)."""
+    import lvar_amd.torch_ops as tops
+    tops.register_as("chipmunk")
+    g = torch.Generator().manual_seed(31)
+    mask = torch.rand(2, 3, 5, 300, generator=g) < 0.3
+    mask[0, 0, 0] = False
+    mask[0, 0, 1] = True
+    for ns in (torch.ops.lvar, torch.ops.chipmunk):
+        for mult, pad_to in ((1, 192), (64, 192), (7, 1)):
+            indices, counts = ns.mask_to_indices(mask.cuda(), mult, pad_to)
+            pad_n = (300 + pad_to - 1) // pad_to * pad_to
+            assert indices.dtype == torch.int32 and tuple(indices.shape) == (2, 3, 5, pad_n) and tuple(counts.shape) == (2, 3, 5)
+            c_ref, i_ref = oracle.mask_to_lists(mask, mult)
+            assert torch.equal(counts.cpu(), c_ref) and torch.equal(indices[..., :300].cpu(), i_ref)
+        with pytest.raises(Exception):
+            ns.mask_to_indices(mask.cuda().to(torch.uint8), 1, 192)          # "mask must be bool type"
+        with pytest.raises(Exception):
+            ns.mask_to_indices(mask.cuda()[0], 1, 192)                        # "mask must be 4-dimensional"
+    act = torch.randn(2, 4, 1000, generator=g)
+    act[0, 0, 100:200] = 0.25                                                 # ties through the cut
+    for ns in (torch.ops.lvar, torch.ops.chipmunk):
+        for dtype in (torch.float32, torch.bfloat16):
+            a = act.to(dtype)
+            for sparsity, mult in ((0.8, 8), (0.75, 64), (0.0, 1), (0.5, 1)):
+                indices = torch.full((2, 4, 1000), -1, dtype=torch.int32, device="cuda")
+                counts = torch.zeros(2, 4, dtype=torch.int32, device="cuda")
+                assert ns.topk_indices(a.cuda(), indices, counts, sparsity, mult, 0.0) is None
+                keep = 1000 - int(1000 * sparsity)
+                padded = min(1000, (keep + mult - 1) // mult * mult)
+                assert bool((counts == padded).all())
+                top = oracle.topk_token_set(a.float(), keep)                   # stable selection, ascending
+                sel = torch.zeros(2, 4, 1000, dtype=torch.bool).scatter_(-1, top.long(), True)
+                c_ref, i_ref = oracle.mask_to_lists(sel, mult)                 # + the lowest unselected columns as padding
+                assert torch.equal(counts.cpu(), c_ref) and torch.equal(indices[..., :padded].cpu(), i_ref[..., :padded])
+                assert bool((indices[..., padded:] == -1).all())                # left as the caller filled them
+        indices = torch.zeros(2, 4, 1000, dtype=torch.int32, device="cuda")
+        counts = torch.ones(2, 4, dtype=torch.int32, device="cuda")
+        ns.topk_indices(act.cuda(), indices, counts, 1.0, 8, 0.0)               # quantile 1: no indices
+        assert bool((indices == -1).all()) and bool((counts == 0).all())
+        # random extras: the top set stays, every count is a multiple, lists are free of repeats
+        indices.fill_(-1)
+        ns.topk_indices(act.cuda(), indices, counts, 0.9, 16, 0.2)
+        top = oracle.topk_token_set(act, 100)
+        for b in range(2):
+            for r in range(4):
+                c = int(counts[b, r])
+                row = indices[b, r, :c].cpu()
+                assert c % 16 == 0 and c >= 112 and len(set(row.tolist())) == c and int(row.min()) >= 0 and int(row.max()) < 1000
+                assert set(top[b, r].tolist()) <= set(row.tolist())
+        with pytest.raises(Exception):
+            ns.topk_indices(act.cuda(), indices, counts, 1.5, 8, 0.0)
 
 
 def test_sparse_diff_attn_full_and_sparse_steps():

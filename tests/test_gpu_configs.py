@@ -67,7 +67,7 @@ def test_colsum_config_block_sums_and_topk(Lq, Lk):
 
 # ---------------------------------------------------------------- density sweep
 
-@pytest.mark.parametrize("pct", [5, 25, 75])
+@pytest.mark.parametrize("pct", [5, 10, 25, 50, 75])
 def test_density_sweep_full_size(pct):
     """B1 H16 Lq4096 Lk10521, 128x64 blocks, Bernoulli(pct) block masks with at least one block per row."""
     from lvar_amd import mask_build as mb, sparse_attn_ops as ops

@@ -36,13 +36,14 @@ def test_kernel_config_and_yaml_merge():
         cfg.get_kernel_config_attn()
 
 
-def test_topk_index_list_matches_oracle():
+def test_list_builders_have_no_cpu_path():
+    """The top-k list and the block-list compaction are HIP kernels: host tensors are refused, not served by torch
+    (the GPU tests compare them with the oracle).  Argument errors are still reported before the device is looked at."""
     bs = torch.rand(2, 3, 4, 680, generator=torch.Generator().manual_seed(0))
-    inds, counts = mb.topk_index_list(bs, 0.5)
-    oi, oc = oracle.topk_index_list(bs, 0.5)
-    assert int(counts[0, 0, 0]) == 320 and torch.equal(counts, oc)
-    assert inds.shape == (2, 3, 4, 680) and inds.dtype == torch.int32
-    assert torch.equal(inds[..., :320], oi[..., :320])
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mb.topk_index_list(bs, 0.5)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mb.block_mask_to_lists(bs > 0.5)
     with pytest.raises(ValueError):
         mb.topk_index_list(bs[..., :10], 7.0)
 
@@ -98,18 +99,12 @@ def test_flex_block_mask_matches_oracle():
     assert m.shape == (32, 83) and bool(m[:, 0].all())
 
 
-def test_block_lists_and_sums_match_oracle():
-    mask = torch.rand(2, 3, 5, 17, generator=torch.Generator().manual_seed(3)) < 0.3
-    n1, i1 = mb.block_mask_to_lists(mask)
-    n2, i2 = oracle.block_mask_to_lists(mask)
-    assert torch.equal(n1, n2) and torch.equal(i1, i2) and i1.dtype == torch.int32
-    assert torch.equal(oracle.lists_to_block_mask(n1, i1, 17), mask)
+def test_block_sums_and_keep_counts():
     cs = torch.rand(1, 2, 3, 680, generator=torch.Generator().manual_seed(4))
     assert torch.allclose(mb.key_block_sums(cs, 64), oracle.key_block_sums(cs, 64))
-    num, idx = mb.topk_block_lists(mb.key_block_sums(cs, 64), 0.5, k_len=680)
-    assert int(num[0, 0, 0]) == 5                              # 64*round(0.5*680/64)/64, VAR-d16 benchmark case
-    assert int(mb.topk_block_lists(mb.key_block_sums(cs, 64), 0.5)[0][0, 0, 0]) == 6   # round(5.5), half-to-even
-    assert bool((idx[..., 1:] > idx[..., :-1]).all())
+    assert mb.block_keep_count(0.5, 11, k_len=680) == 5       # 64*round(0.5*680/64)/64, VAR-d16 benchmark case
+    assert mb.block_keep_count(0.5, 11) == 6                  # round(5.5), half-to-even
+    assert mb.block_keep_count(0.0, 11) == 1 and mb.block_keep_count(3.0, 11) == 11
 
 
 def test_sink_window_topk_mask_matches_oracle():

@@ -194,6 +194,24 @@ def test_local_window_runs_known_answers():
         assert tuple(runs.shape) == shape and L == shape[1]
         assert bool((runs[:, 1:] - runs[:, :-1] == 1).all())                  # contiguous runs
         assert int(runs.min()) >= oracle.infinity_cum()[si] and int(runs.max()) == kv - 1
+    # Run starts worked out by hand (sparse_attn.py:845-855).  Scale 11 (48 x 48 grid at key 4121, Lk 6425), window 5,
+    # 192-row groups = grid rows 4g..4g+3: the union of the clamped windows is the full rows max(4g-2, 0)..min(4g+5, 47),
+    # i.e. first key 4121 + 48 * max(4g-2, 0) and 288 or 384 keys -> 448 after rounding up to a multiple of 112; the run
+    # is [first, first + 447], pushed back to end at key 6424 for the last groups.
+    # Scale 12 (64 x 64 grid at key 6425, Lk 10521), window 7, groups = grid rows 3g..3g+2 (the last group is row 63
+    # alone): rows max(3g-3, 0)..min(3g+5, 63), at most 576 keys -> 672; first key 6425 + 64 * max(3g-3, 0).
+    from lvar_amd import mask_build as mb
+    hand = {(11, 5): {0: 4121, 1: 4217, 5: 4985, 10: 5945, 11: 5977},
+            (12, 7): {0: 6425, 1: 6425, 2: 6617, 10: 8153, 20: 9849, 21: 9849}}
+    for (si, win), starts in hand.items():
+        ia, kv = oracle.crossscale_self_indices(si, win)
+        S = oracle.INFINITY_SCALES[si]
+        runs, L = oracle.aggregate_group_indices(ia, S * S, kv, 192, 112)
+        runs_mb, L_mb = mb.local_group_runs(si, win, 192, 112)
+        assert L_mb == L and torch.equal(runs_mb.cpu().to(torch.int64), runs)
+        for g, first in starts.items():
+            assert int(runs[g, 0]) == first and int(runs[g, -1]) == first + L - 1, (si, g)
+            assert int(runs_mb[g, 0]) == first, (si, g)
     # interior query of an 8x8 grid, 3x3 window: the 9 neighbours, row-major
     w = oracle.local_window_indices(8, 8, 100, 3)
     assert w[9].tolist() == [100, 101, 102, 108, 109, 110, 116, 117, 118]

@@ -87,3 +87,9 @@ def test_static_scratch_limits():
                                                ng.data_ptr(), 0, 0, ig.data_ptr(), 0, 0, ig.stride(2), ig.shape[3],
                                                128, 64, big_B, 2, 256, 512, 128, 0.1, ops._stream(fake_q))
     assert st == -4 and b"static scratch" in lib.lvar_status_string(st)
+    # arguments are checked before the scratch is looked at: the same refusals as the workspace entry point
+    for (bq, scale, want) in ((96, 0.1, -2), (128, -1.0, -1)):
+        st = lib.lvar_block_sparse_attn_static_fwd(ops._view(qg), ops._view(kg), ops._view(vg), ops._view(torch.empty_like(qg)), M.data_ptr(), M.data_ptr(),
+                                                   ng.data_ptr(), 0, 0, ig.data_ptr(), 0, 0, ig.stride(2), ig.shape[3],
+                                                   bq, 64, 1, 2, 256, 512, 128, scale, ops._stream(qg))
+        assert st == want
