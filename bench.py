@@ -384,51 +384,13 @@ def run_hbm_workload(args, dev, wl):
         "cpu_baseline": cpu, "device": torch.cuda.get_device_name(0)}))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="block_sparse_25",
-                    help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | full_step | density_<pct> | video_10 | infinity2b_schedule | topk_tokens | remap_lists | window_scores | copy_1gib")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-aux", action="store_true", help="skip the companion dense/colsum/mask-build timings")
-    ap.add_argument("--cpu-budget-s", type=float, default=12.0)
-    ap.add_argument("--settle-ms", type=float, default=150.0,
-                    help="untimed load run before the warm-up steps so that the clocks have settled (0 = off)")
-    ap.add_argument("--amp", type=float, default=None, help="override the input amplitude (0 = all-zero inputs, for power experiments)")
-    args = ap.parse_args()
-    global SETTLE_MS
-    SETTLE_MS = args.settle_ms
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs the hot path on ONE GPU; --gpus N with N > 1 is not supported "
-              "(the path shards over (batch, head) with no exchange step: give every GPU its own heads).", file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU (no CPU fallback)", file=sys.stderr)
-        sys.exit(1)
-
+def setup_workload(wl, args, dev, want_cpu, want_parts):
+    """Inputs, launch closure, algorithmic flops and description of one attention / colsum workload.  ``want_cpu``:
+    also time the oracle on the host cores; ``want_parts``: also time the workload's component kernels."""
     from lvar_amd import mask_build as mb
     from lvar_amd import sparse_attn_ops as ops
-
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    wl = args.workload
-    if wl in ("topk_tokens", "remap_lists", "window_scores"):
-        run_hbm_workload(args, dev, wl)
-        return
-    if wl == "infinity2b_schedule":
-        run_infinity_schedule(args, dev)
-        return
-    if wl == "copy_1gib":
-        # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
-        x = torch.empty(1 << 28, dtype=torch.float32, device=dev)
-        y = torch.empty_like(x)
-        ms, _ = time_launches(lambda: y.copy_(x), args.steps, args.warmup)
-        print(json.dumps({"metric": "device copy bandwidth", "value": round(2 * x.numel() * 4 / ms / 1e6, 1), "unit": "GB/s",
-                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
-                          "config": {"workload": wl, "bytes_read": x.numel() * 4, "bytes_written": x.numel() * 4}}))
-        return
+    dense_ms = None
+    num = idx = None
     d = 128
     aux = {}
     cpu = None
@@ -479,14 +441,14 @@ def main():
         config["active_block_fraction"] = round(float(num.float().mean().item()) / nK, 4)
         fn = lambda: ops.block_sparse_attn(qg, kg, vg, num, idx, bq, bk, scale)
         kernel = "attn_fwd_kernel<128,4,MODE_BLOCK>"
-        if not args.no_cpu_baseline:
+        if want_cpu:
             val, sample = cpu_baseline_block_sparse(q, k, v, num.cpu(), idx.cpu(), bq, bk, args.cpu_budget_s)
             cpu = {"value": round(val, 5), "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port", "sample": sample}
     elif wl == "dense":
         flops = dense_flops
         fn = lambda: ops.dense_attn(qg, kg, vg, scale)
         kernel = "attn_fwd_kernel<128,4,MODE_BLOCK> (identity list)"
-        if not args.no_cpu_baseline:
+        if want_cpu:
             done, t = cpu_baseline_dense(q, k, v, args.cpu_budget_s)
             cpu = {"value": round(dense_flops / (B * H) * done / t / 1e12, 5), "unit": "TFLOP/s", "cores": os.cpu_count(),
                    "kind": "port", "sample": f"{done} (batch,head) slices (the workload has {B * H}; cycled), {t:.1f} s of host time"}
@@ -496,7 +458,7 @@ def main():
         fn = lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 192)
         kernel = "colsum_kernel<128>"
         config["form"] = "one-pass given (M,L): 2*B*H*Lq*Lk*d flops"
-        if not args.no_cpu_baseline:
+        if want_cpu:
             done, t = cpu_baseline_dense(q, k, v, args.cpu_budget_s, colsum=True)
             cpu = {"value": round(1.5 * dense_flops / (B * H) * done / t / 1e12, 5), "unit": "TFLOP/s", "cores": os.cpu_count(),
                    "kind": "port", "sample": f"{done} (batch,head) slices (the workload has {B * H}; cycled) of dense attention + colsum (6*Lq*Lk*d flops each), {t:.1f} s of host time"}
@@ -516,10 +478,12 @@ def main():
         o_d, _, _, _ = ops._dense_launch(qg, kg, vg, scale)
         cs = ops._colsum_given_lse(qg, kg, lse2, scale, 192)
         i_d, c_d = mb.topk_index_list(cs, 0.2, order="index")
-        parts = {"dense_attn_us": dense_ms * 1e3,
-                 "colsum_us": time_launches(lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 192), 20, 5)[0] * 1e3,
-                 "topk_lists_us": time_launches(lambda: mb.topk_index_list(cs, 0.2, order="index"), 20, 5)[0] * 1e3,
-                 "ocache_csp_us": time_launches(lambda: ops.csp_attn(qg, kg, vg, scale, i_d, c_d, o_d, -1), 20, 5)[0] * 1e3}
+        parts = {"dense_attn_us": dense_ms * 1e3}
+        if want_parts:
+            parts.update({
+                "colsum_us": time_launches(lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 192), 20, 5)[0] * 1e3,
+                "topk_lists_us": time_launches(lambda: mb.topk_index_list(cs, 0.2, order="index"), 20, 5)[0] * 1e3,
+                "ocache_csp_us": time_launches(lambda: ops.csp_attn(qg, kg, vg, scale, i_d, c_d, o_d, -1), 20, 5)[0] * 1e3})
         aux = {k_: round(v_, 1) for k_, v_ in parts.items()}
         config.update({"top_keys": 0.2, "decision_scale": 10, "count": int(c_d[0, 0, 0])})
     elif wl == "csp":
@@ -527,7 +491,7 @@ def main():
         cs = ops.colsum(qg, kg, scale)
         inds, counts = mb.topk_index_list(cs, 0.2, order="index")     # GPU radix select, ascending key order
         cnt = int(counts[0, 0, 0])
-        if not args.no_aux:
+        if want_parts:
             topk_ms, _ = time_launches(lambda: ops.topk_token_lists(cs, cnt), 10, 3)
             torch_ms, _ = time_launches(lambda: torch.topk(cs, cnt, dim=-1), 5, 2)
             ref_set = torch.topk(cs, cnt, dim=-1).indices.sort(-1).values
@@ -541,31 +505,180 @@ def main():
         kernel = "attn_fwd_kernel<128,6,MODE_GATHER>"
         config.update({"top_keys": 0.2, "count": cnt})
 
+    return {"fn": fn, "flops": flops, "kernel": kernel, "config": config, "cpu": cpu, "aux": aux, "amp": amp, "dense_ms": dense_ms,
+            "q": qg, "k": kg, "v": vg, "scale": scale, "num": num, "idx": idx, "dense_flops": dense_flops}
+
+
+def headline_companions(w, ms):
+    """The numbers the metric names beside the block-sparse rate: colsum and the GPU mask build against the dense
+    attention they replace, in the form that reuses the row statistics of a dense pass (given ``lse2``) and in the
+    self-contained two-pass form (statistics sweep + column sweep)."""
+    from lvar_amd import mask_build as mb
+    from lvar_amd import sparse_attn_ops as ops
+    qg, kg, vg, scale, num, idx = w["q"], w["k"], w["v"], w["scale"], w["num"], w["idx"]
+    dense_ms, _ = time_launches(lambda: ops.dense_attn(qg, kg, vg, scale), 10, 3)
+    lse2 = ops._lse_only(qg, kg, scale)
+    cs_ms, _ = time_launches(lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 128), 10, 3)
+    lse_ms, _ = time_launches(lambda: ops._lse_only(qg, kg, scale), 10, 3)
+    base = mb.sink_window_base_mask(128, 64, device=qg.device)
+    target = int(round(0.25 * base.shape[1]))
+
+    def build():
+        _, bs = ops._colsum_given_lse(qg, kg, lse2, scale, 128, want_block_sums=True)
+        return ops.block_topk_lists(bs, target, base)
+
+    def build_two_pass():
+        _, bs = ops.colsum(qg, kg, scale, q_group_size=128, return_block_sums=True)
+        return ops.block_topk_lists(bs, target, base)
+    n2, i2 = build()
+    assert torch.equal(n2, num) and torch.equal(i2, idx), "GPU list build differs from the torch selection"
+    n3, i3 = build_two_pass()
+    assert torch.equal(n3, num) and torch.equal(i3, idx), "two-pass GPU list build differs from the torch selection"
+    build_ms, _ = time_launches(build, 5, 2)
+    build2_ms, _ = time_launches(build_two_pass, 5, 2)
+    return {"dense_attn_ms": round(dense_ms, 4), "dense_attn_tflops": round(w["dense_flops"] / dense_ms / 1e9, 1),
+            "colsum_given_lse_us": round(cs_ms * 1e3, 1), "lse_pass_us": round(lse_ms * 1e3, 1),
+            "colsum_plus_mask_build_ms": round(build_ms, 4),
+            "colsum_plus_mask_build_two_pass_ms": round(build2_ms, 4),
+            "colsum_plus_mask_build_over_dense": round(build_ms / dense_ms, 3),
+            "colsum_plus_mask_build_two_pass_over_dense": round(build2_ms / dense_ms, 3),
+            "speedup_vs_dense": round(dense_ms / ms, 3)}
+
+
+def colsum_config(args, dev, Lq, Lk):
+    """BASELINE configuration 3: the colsum kernel alone at one scale (B2 H16 d128, N(0,1) inputs, 192-row groups),
+    its per-64-key block sums and the block top-k lists at keep ratios 10 / 25 / 50 %; given the row statistics of a
+    dense pass, and self-contained (statistics sweep + column sweep)."""
+    from lvar_amd import sparse_attn_ops as ops
+    B, H, d = 2, 16, 128
+    q, k, _ = make_qkv(B, H, Lq, Lk, d, seed=1234, amp=1.0)
+    qg, kg = q.to(dev), k.to(dev)
+    scale = 1.0 / math.sqrt(d)
+    lse2 = ops._lse_only(qg, kg, scale)
+    flops = 2.0 * B * H * Lq * Lk * d
+    st, wu = max(5, args.steps // 3), max(3, args.warmup // 4)
+    cs_ms, _ = time_launches(lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 192, want_block_sums=True), st, wu)
+    two_ms, _ = time_launches(lambda: ops.colsum(qg, kg, scale, q_group_size=192, return_block_sums=True), st, wu)
+    _, bs = ops._colsum_given_lse(qg, kg, lse2, scale, 192, want_block_sums=True)
+    out = {"Lq": Lq, "Lk": Lk, "colsum_given_lse_us": round(cs_ms * 1e3, 1), "tflops": round(flops / cs_ms / 1e9, 1),
+           "frac": round(flops / cs_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+           "colsum_two_pass_us": round(two_ms * 1e3, 1), "two_pass_tflops": round(2 * flops / two_ms / 1e9, 1),
+           "two_pass_frac": round(2 * flops / two_ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    nK = bs.shape[-1]
+    for keep in (10, 25, 50):
+        target = int(round(keep / 100.0 * nK))
+        t_ms, _ = time_launches(lambda: ops.block_topk_lists(bs, target), st, wu)
+        out[f"block_topk_{keep}pct_us"] = round(t_ms * 1e3, 1)
+    return out
+
+
+def other_configs(args, dev):
+    """The benchmark configurations beside the headline one, each timed in this run with fewer steps: density sweep
+    against dense attention on the same shape (configuration 4), long-video block-sparse attention (5), colsum alone
+    at scales 48 and 64 (3), and the two steps of the column-sparse caller (token-list attention at the last scale,
+    the full decision-scale step)."""
+    st, wu = max(5, args.steps // 3), max(3, args.warmup // 4)
+    out = {"steps": st, "warmup": wu}
+
+    def one(wl, parts=False):
+        w = setup_workload(wl, args, dev, want_cpu=False, want_parts=parts)
+        ms, _ = time_launches(w["fn"], st, wu)
+        tf = w["flops"] / ms / 1e9
+        r = {"us": round(ms * 1e3, 1), "tflops": round(tf, 1), "frac": round(tf / PEAK_BF16_TFLOPS, 4)}
+        if "active_block_fraction" in w["config"]:
+            r["active_block_fraction"] = w["config"]["active_block_fraction"]
+        return r, w, ms
+    sweep = {}
+    for pct in (5, 10, 25, 50, 75, 100):
+        r, w, ms = one(f"density_{pct}")
+        if pct == 100:
+            from lvar_amd import sparse_attn_ops as ops
+            d_ms, _ = time_launches(lambda: ops.dense_attn(w["q"], w["k"], w["v"], w["scale"]), st, wu)
+            sweep["dense_same_shape"] = {"us": round(d_ms * 1e3, 1), "tflops": round(w["dense_flops"] / d_ms / 1e9, 1)}
+        sweep[str(pct)] = r
+        del w
+    for pct in (5, 10, 25, 50, 75, 100):
+        sweep[str(pct)]["vs_dense_tflops"] = round(sweep[str(pct)]["tflops"] / sweep["dense_same_shape"]["tflops"], 3)
+    out["density_sweep_B1"] = sweep
+    torch.cuda.empty_cache()
+    out["video_10"], w, _ = one("video_10")
+    del w
+    torch.cuda.empty_cache()
+    out["colsum_scale48"] = colsum_config(args, dev, 2304, 6425)
+    out["colsum_scale64"] = colsum_config(args, dev, 4096, 10521)
+    out["csp_top20pct_last_scale"], w, _ = one("csp")
+    del w
+    r, w, ms = one("full_step", parts=True)
+    r.update(w["aux"])
+    r["full_step_over_dense"] = round(ms / w["dense_ms"], 3)
+    r.pop("tflops"), r.pop("frac")
+    out["full_step_decision_scale"] = r
+    del w
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="block_sparse_25",
+                    help="block_sparse_25 (headline) | dense | colsum | colsum_scale48 | csp | full_step | density_<pct> | video_10 | infinity2b_schedule | topk_tokens | remap_lists | window_scores | copy_1gib")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-aux", action="store_true", help="skip the companion dense/colsum/mask-build timings")
+    ap.add_argument("--cpu-budget-s", type=float, default=12.0)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed load run before the warm-up steps so that the clocks have settled (0 = off)")
+    ap.add_argument("--amp", type=float, default=None, help="override the input amplitude (0 = all-zero inputs, for power experiments)")
+    args = ap.parse_args()
+    global SETTLE_MS
+    SETTLE_MS = args.settle_ms
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the hot path on ONE GPU; --gpus N with N > 1 is not supported "
+              "(the path shards over (batch, head) with no exchange step: give every GPU its own heads).", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU fallback)", file=sys.stderr)
+        sys.exit(1)
+
+    from lvar_amd import mask_build as mb
+    from lvar_amd import sparse_attn_ops as ops
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    wl = args.workload
+    if wl in ("topk_tokens", "remap_lists", "window_scores"):
+        run_hbm_workload(args, dev, wl)
+        return
+    if wl == "infinity2b_schedule":
+        run_infinity_schedule(args, dev)
+        return
+    if wl == "copy_1gib":
+        # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
+        x = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+        y = torch.empty_like(x)
+        ms, _ = time_launches(lambda: y.copy_(x), args.steps, args.warmup)
+        print(json.dumps({"metric": "device copy bandwidth", "value": round(2 * x.numel() * 4 / ms / 1e6, 1), "unit": "GB/s",
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+                          "config": {"workload": wl, "bytes_read": x.numel() * 4, "bytes_written": x.numel() * 4}}))
+        return
+    w = setup_workload(wl, args, dev, want_cpu=not args.no_cpu_baseline, want_parts=not args.no_aux)
+    fn, flops, aux, cpu, kernel, config, amp = w["fn"], w["flops"], w["aux"], w["cpu"], w["kernel"], w["config"], w["amp"]
     ms, wall_ms = time_launches(fn, args.steps, args.warmup)
     tflops = flops / (ms * 1e-3) / 1e12
     single = per_launch_stats(fn)
-
-    if wl == "block_sparse_25" and not args.no_aux:
-        # companion numbers named by the metric: colsum (+ mask build) versus the dense attention it replaces
-        dense_ms, _ = time_launches(lambda: ops.dense_attn(qg, kg, vg, scale), 10, 3)
-        lse2 = ops._lse_only(qg, kg, scale)
-        cs_ms, _ = time_launches(lambda: ops._colsum_given_lse(qg, kg, lse2, scale, 128), 10, 3)
-        lse_ms, _ = time_launches(lambda: ops._lse_only(qg, kg, scale), 10, 3)
-
-        base = mb.sink_window_base_mask(128, 64, device=dev)
-        target = int(round(0.25 * base.shape[1]))
-
-        def build():
-            _, bs = ops._colsum_given_lse(qg, kg, lse2, scale, 128, want_block_sums=True)
-            return ops.block_topk_lists(bs, target, base)
-        n2, i2 = build()
-        assert torch.equal(n2, num) and torch.equal(i2, idx), "GPU list build differs from the torch selection"
-        build_ms, _ = time_launches(build, 5, 2)
-        aux = {"dense_attn_ms": round(dense_ms, 4), "dense_attn_tflops": round(dense_flops / dense_ms / 1e9, 1),
-               "colsum_given_lse_us": round(cs_ms * 1e3, 1), "lse_pass_us": round(lse_ms * 1e3, 1),
-               "colsum_plus_mask_build_ms": round(build_ms, 4), "speedup_vs_dense": round(dense_ms / ms, 3)}
-
+    if wl == "full_step":
+        aux["full_step_us"] = round(ms * 1e3, 1)
+        aux["full_step_over_dense"] = round(ms / w["dense_ms"], 3)
     probe = None if args.no_aux else sustained_mfma_rate()
+    if wl == "block_sparse_25" and not args.no_aux:
+        # the numbers the metric names beside the block-sparse rate, then the other benchmark configurations
+        aux.update(headline_companions(w, ms))
+        del w, fn
+        torch.cuda.empty_cache()
+        aux["configs"] = other_configs(args, dev)
+
     traffic, traffic_src = measured_traffic(wl)
     dev_sum = device_summary()
     # CU count x 4096 flop per clock x maximum engine clock, as the device reports them at run time; `peak` and
@@ -588,9 +701,6 @@ def main():
         "cpu_baseline": cpu,
         "device": torch.cuda.get_device_name(0), "device_summary": dev_sum,
     }
-    if wl == "full_step":
-        aux["full_step_us"] = round(ms * 1e3, 1)
-        aux["full_step_over_dense"] = round(ms / dense_ms, 3)
     if aux:
         out["aux"] = aux
     print(json.dumps(out))
