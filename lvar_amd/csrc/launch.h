@@ -117,7 +117,7 @@ struct WinScoreParams {
   const int64_t* window;  // [B*H, W] key positions of the window tokens
   float* out;             // [B*H, Lk]
   int64_t q_sb, q_sh, q_sr, k_sb, k_sh, k_sr;
-  int B, H, Lq, Lk, W, ksize, maxpool, nchunks;
+  int B, H, Lq, Lk, W, ksize, maxpool, nchunks, total_wg;
   float scale;
 };
 

@@ -19,7 +19,13 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const WinScoreParams
   __shared__ float sc[WS_KEYS + 2 * WS_MAXR];
   __shared__ uint8_t wm[WS_KEYS + 2 * WS_MAXR];
   const int tid = threadIdx.x;
-  const int bh = blockIdx.x / p.nchunks, chunk = blockIdx.x - bh * p.nchunks;
+  // Workgroup ids are dealt round-robin to the 8 XCDs, each with an L2 of its own; remapped so that one XCD walks a
+  // contiguous range of (batch, head, chunk), the window queries of a (batch, head) are fetched from memory by one
+  // XCD instead of by all eight (they are read by every workgroup of the slice: as many bytes as 256 keys).
+  const int per_xcd = gridDim.x >> 3;
+  const int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (w >= p.total_wg) return;
+  const int bh = w / p.nchunks, chunk = w - bh * p.nchunks;
   const int b = bh / p.H, h = bh - b * p.H;
   const int r = p.ksize >> 1;
   const int n0 = chunk * WS_KEYS - r;  // key of sc[0]
@@ -115,7 +121,8 @@ int launch_window_scores(const WinScoreParams& p0, int head_dim, hipStream_t str
   WinScoreParams p = p0;
   if ((p.ksize & 1) == 0 || p.ksize < 1 || (p.ksize >> 1) > WS_MAXR) return LVAR_EUNSUPPORTED;
   p.nchunks = (p.Lk + WS_KEYS - 1) / WS_KEYS;
-  const dim3 grid(p.B * p.H * p.nchunks);
+  p.total_wg = p.B * p.H * p.nchunks;
+  const dim3 grid((p.total_wg + 7) / 8 * 8);
   if (head_dim == 128) hipLaunchKernelGGL(window_scores_kernel<128>, grid, dim3(256), 0, stream, p);
   else if (head_dim == 64) hipLaunchKernelGGL(window_scores_kernel<64>, grid, dim3(256), 0, stream, p);
   else if (head_dim == 256) hipLaunchKernelGGL(window_scores_kernel<256>, grid, dim3(256), 0, stream, p);

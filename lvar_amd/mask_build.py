@@ -63,10 +63,15 @@ def topk_index_list(bs: torch.Tensor, top_keys: float, multiple_of: Optional[int
 
 
 def map_inds_counts_across_scales(inds_S: torch.Tensor, counts_S, cur_q_len: int, cur_k_len: int,
-                                  bm: int = 192, indices_pad_to: int = 1) -> Tuple[torch.Tensor, torch.Tensor]:
+                                  bm: int = 192, indices_pad_to: int = 1, add_sink: bool = False, sink_len: int = 0,
+                                  sink_quota_frac: float = 0.2) -> Tuple[torch.Tensor, torch.Tensor]:
     """Nearest query-group remap of a key list from the decision scale to the current scale
-    (models/sparvar/sparse_attn.py:366-421, the path without sink).  ``counts_S`` may be a tensor
-    (its [0,0,0] element is read, one host sync as in the reference) or a Python int."""
+    (models/sparvar/sparse_attn.py:366-469).  ``counts_S`` may be a tensor (its [0,0,0] element is read, one host
+    sync as in the reference) or a Python int.  ``add_sink`` (the branch at :423-469, which no shipped
+    configuration switches on): the first ``min(round(count*sink_quota_frac), count, sink_len)`` entries are the keys
+    from 0 on, the others the smallest entries >= ``sink_len`` of the whole source row in ascending order.  The
+    default path also exists as one kernel fused with the local-run append
+    (:func:`lvar_amd.sparse_attn_ops.remap_concat_lists`); the sink path is torch on the lists' device."""
     B, H, Gs, Ks = inds_S.shape
     Gk = (cur_q_len + bm - 1) // bm
     raw = int(counts_S[0, 0, 0]) if torch.is_tensor(counts_S) else int(counts_S)
@@ -74,13 +79,23 @@ def map_inds_counts_across_scales(inds_S: torch.Tensor, counts_S, cur_q_len: int
     centers = torch.arange(Gk, device=inds_S.device, dtype=torch.float32) + 0.5
     src = torch.round(centers / Gk * Gs - 0.5).to(torch.int64).clamp_(0, Gs - 1)
     templ = inds_S.index_select(2, src)
-    if Ks >= cnt:
-        out = templ[..., :cnt].to(torch.int32)
-    else:
-        out = templ.repeat_interleave(math.ceil(cnt / Ks), dim=-1)[..., :cnt].to(torch.int32)
-    out = out.clamp(0, max(0, cur_k_len - 1)).contiguous()
     counts = torch.full((B, H, Gk), cnt, dtype=torch.int32, device=inds_S.device)
-    return out, counts
+    if not add_sink or sink_len <= 0 or cnt == 0:
+        if Ks >= cnt:
+            out = templ[..., :cnt].to(torch.int32)
+        else:
+            out = templ.repeat_interleave(math.ceil(cnt / Ks), dim=-1)[..., :cnt].to(torch.int32)
+        return out.clamp(0, max(0, cur_k_len - 1)).contiguous(), counts
+    sink_quota = min(int(round(cnt * sink_quota_frac)), cnt, sink_len)
+    quota = cnt - sink_quota
+    big = torch.iinfo(torch.int32).max
+    vals = torch.where(templ >= sink_len, templ.to(torch.int64), torch.full_like(templ, big, dtype=torch.int64))
+    vals = vals.sort(dim=-1).values                    # the smallest surviving entries first
+    if quota > Ks:
+        vals = vals.repeat_interleave(math.ceil(quota / Ks), dim=-1)
+    head = torch.arange(sink_quota, device=inds_S.device, dtype=torch.int64).expand(B, H, Gk, sink_quota)
+    out = torch.cat([head, vals[..., :quota]], dim=-1).clamp(0, max(0, cur_k_len - 1)).to(torch.int32)
+    return out.contiguous(), counts
 
 
 def local_group_runs(scale_idx: int, win: int, bm: int = 192, counts_multiple_of: Optional[int] = None,

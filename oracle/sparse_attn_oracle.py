@@ -240,25 +240,47 @@ def lists_to_block_mask(num, idx, nK):
     return mask
 
 
-def map_inds_counts_across_scales(inds_S, counts_S, cur_q_len, cur_k_len, bm=192, indices_pad_to=1):
-    """Query-group remap between scales, the path without sink
-    (models/sparvar/sparse_attn.py:366-421): ``gS = clamp(round((g+0.5)/Gk*Gs - 0.5), 0, Gs-1)``
-    with float32 arithmetic and round-half-to-even (torch.round), first ``indices_count``
-    columns (cyclic ``repeat_interleave`` when the source is narrower), clamp to [0, Lk-1]."""
+def map_inds_counts_across_scales(inds_S, counts_S, cur_q_len, cur_k_len, bm=192, indices_pad_to=1,
+                                  add_sink=False, sink_len=0, sink_quota_frac=0.2):
+    """Query-group remap between scales (models/sparvar/sparse_attn.py:366-469):
+    ``gS = clamp(round((g+0.5)/Gk*Gs - 0.5), 0, Gs-1)`` with float32 arithmetic and round-half-to-even (torch.round).
+    Without sink (:412-421): the first ``indices_count`` columns of the source row (cyclic ``repeat_interleave`` when
+    the source is narrower), clamped to [0, Lk-1].
+    With sink (:423-469): the first ``sink_quota = min(round(indices_count*frac), indices_count, sink_len)`` columns
+    are the keys 0 .. sink_quota-1; the rest are the smallest entries >= ``sink_len`` of the WHOLE source row, in
+    ascending order (entries below ``sink_len`` count as int32 max, so a row with too few large entries is filled up
+    with that value; when the quota exceeds the row width every pick is repeated ``ceil(quota/Ks)`` times in place);
+    then the clamp.  Pure-Python loops over rows."""
     B, H, Gs, Ks = inds_S.shape
     Gk = (cur_q_len + bm - 1) // bm
     raw = int(counts_S[0, 0, 0])
     cnt = max(indices_pad_to, (raw + indices_pad_to - 1) // indices_pad_to * indices_pad_to)
     out = torch.empty(B, H, Gk, cnt, dtype=torch.int32)
+    sink = bool(add_sink) and sink_len > 0 and cnt > 0
+    sink_quota = min(int(round(cnt * sink_quota_frac)), cnt, sink_len) if sink else 0
+    big = int(np.iinfo(np.int32).max)
     for g in range(Gk):
         u = np.float32(np.float32(np.float32(g) + np.float32(0.5)) / np.float32(Gk)) * np.float32(Gs) - np.float32(0.5)
         gs = int(np.clip(np.rint(np.float32(u)), 0, Gs - 1))  # np.rint is half-to-even
         row = inds_S[:, :, gs]
-        if Ks >= cnt:
-            out[:, :, g] = row[..., :cnt]
-        else:
-            rep = math.ceil(cnt / Ks)
-            out[:, :, g] = row.repeat_interleave(rep, dim=-1)[..., :cnt]
+        if not sink:
+            if Ks >= cnt:
+                out[:, :, g] = row[..., :cnt]
+            else:
+                rep = math.ceil(cnt / Ks)
+                out[:, :, g] = row.repeat_interleave(rep, dim=-1)[..., :cnt]
+            continue
+        quota = cnt - sink_quota
+        for b in range(B):
+            for h in range(H):
+                vals = sorted(int(x) if int(x) >= sink_len else big for x in row[b, h].tolist())
+                if quota <= Ks:
+                    pick = vals[:quota]
+                else:
+                    rep = math.ceil(quota / Ks)
+                    pick = [x for x in vals for _ in range(rep)][:quota]
+                full = list(range(sink_quota)) + pick
+                out[b, h, g] = torch.tensor([min(x, big) for x in full], dtype=torch.int64).clamp(max=big).to(torch.int32)
     out.clamp_(0, max(0, cur_k_len - 1))
     counts = torch.full((B, H, Gk), cnt, dtype=torch.int32)
     return out, counts

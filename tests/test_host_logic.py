@@ -62,6 +62,31 @@ def test_map_inds_counts_matches_oracle():
     assert torch.equal(a, b)
 
 
+def test_map_inds_counts_with_sink_matches_oracle_and_hand_case():
+    """The ``add_sink`` branch (models/sparvar/sparse_attn.py:423-469): torch mirror against the brute-force oracle on
+    random lists, and one row worked out by hand."""
+    g = torch.Generator().manual_seed(6)
+    for (Ks, count, pad, sink_len, frac, q_len, k_len) in ((300, 100, 4, 21, 0.2, 2304, 6425), (40, 96, 1, 5, 0.5, 960, 30),
+                                                             (64, 64, 64, 200, 0.2, 192, 4121), (50, 10, 1, 3, 1.0, 400, 77)):
+        inds_S = torch.randint(0, 400, (2, 2, 9, Ks), generator=g, dtype=torch.int32)
+        a, ac = mb.map_inds_counts_across_scales(inds_S, count, q_len, k_len, indices_pad_to=pad, add_sink=True,
+                                                 sink_len=sink_len, sink_quota_frac=frac)
+        b, bc = oracle.map_inds_counts_across_scales(inds_S, torch.tensor([[[count]]]), q_len, k_len, indices_pad_to=pad,
+                                                     add_sink=True, sink_len=sink_len, sink_quota_frac=frac)
+        assert torch.equal(a, b) and torch.equal(ac, bc) and a.dtype == torch.int32
+    # one source group, count 6, sink_len 3, frac 0.5: sink quota min(round(3.0), 6, 3) = 3 -> keys 0, 1, 2; then the three
+    # smallest entries >= 3 of the whole row [7, 1, 9, 3, 3, 50, 2, 8] -> 3, 3, 7; key 50 would be clamped to Lk - 1 = 9
+    row = torch.tensor([7, 1, 9, 3, 3, 50, 2, 8], dtype=torch.int32).view(1, 1, 1, 8)
+    for fn in (mb.map_inds_counts_across_scales, oracle.map_inds_counts_across_scales):
+        out, cnt = fn(row, torch.tensor([[[6]]]), 192, 10, add_sink=True, sink_len=3, sink_quota_frac=0.5)
+        assert out.tolist() == [[[[0, 1, 2, 3, 3, 7]]]] and int(cnt[0, 0, 0]) == 6
+        out, _ = fn(row, torch.tensor([[[8]]]), 192, 10, add_sink=True, sink_len=3, sink_quota_frac=0.25)
+        assert out.tolist() == [[[[0, 1, 3, 3, 7, 8, 9, 9]]]]           # sink quota 2; the six survivors 3, 3, 7, 8, 9, 50, the last clamped to Lk - 1
+        # sink_len 0 or add_sink False: the plain path
+        out, _ = fn(row, torch.tensor([[[4]]]), 192, 10, add_sink=True, sink_len=0)
+        assert out.tolist() == [[[[7, 1, 9, 3]]]]
+
+
 @pytest.mark.parametrize("si,win,m", [(11, 5, 112), (12, 7, 112), (11, 7, 64), (12, 9, 64), (10, 3, 64)])
 def test_local_group_runs_matches_oracle(si, win, m):
     runs, L = mb.local_group_runs(si, win, 192, m)
