@@ -115,6 +115,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
   const int32_t* list = nullptr;
   int T, count;
   int tile0 = 0;   // identity list of a balanced launch: first tile of this piece
+  int avail = 0;   // entries of the list row from `list` on (token lists)
   // first four entries of a block list, read together with the count (not after it): one memory
   // round trip less before the first tile can be fetched; entries beyond the count are never used
   int head[4] = {0, 0, 0, 0};
@@ -131,6 +132,7 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
         if (first + i < p.list_len) head[i] = list[first + i];
     }
     count = max(0, min(p.cnt[b * p.cnt_sb + h * p.cnt_sh + g], p.list_len));
+    avail = p.list_len - first;
     if (SK) {
       const int last = (MODE == MODE_BLOCK) ? u1 : (u1 << 6);
       count = max(0, min(count, last) - first);
@@ -178,11 +180,13 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       if (MODE == MODE_BLOCK) {
         raw[0] = identity ? t + tile0 : list[t >> sub_shift];
       } else {
+        // bounded by the row of the list, not by the count: entries behind the count are never used (they are
+        // clamped and masked), and the read then does not have to wait for the count to arrive
 #pragma unroll
         for (int s = 0; s < SLOTS; s++) {
           const int trow = (fwave + s * FW) * RPI + lrow;
           const int pos = (t << 6) + trow;
-          raw[s] = (pos < count && trow < 64) ? list[pos] : 0;
+          raw[s] = (pos < avail && trow < 64) ? list[pos] : 0;
         }
       }
     };
@@ -259,11 +263,15 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
       int nv_unused;
 #pragma unroll
       for (int s = 0; s < NR; s++) { rows_v[s] = 0; rows_k[s] = 0; rows_n[s] = 0; raw[s] = 0; }
-      prefetch_raw(0, raw);
-      finish_rows(0, raw, rows0, nv_unused);
-      if (T > 1) { prefetch_raw(1, raw); finish_rows(1, raw, rows_v, nv_unused); }
-      if (T > 2) { prefetch_raw(2, raw); finish_rows(2, raw, rows_k, nv_unused); }
-      if (T > 3) prefetch_raw(3, raw);
+      // the list entries of the first four tiles are requested together (one memory round trip, not one per tile)
+      int raw0[NR], raw1[NR], raw2[NR];
+      prefetch_raw(0, raw0);
+      prefetch_raw(1, raw1);
+      prefetch_raw(2, raw2);
+      prefetch_raw(3, raw);
+      finish_rows(0, raw0, rows0, nv_unused);
+      finish_rows(1, raw1, rows_v, nv_unused);
+      finish_rows(2, raw2, rows_k, nv_unused);
       issue(krsrc, k_srb, false, rows0, lds0);
       issue(vrsrc, v_srb, true, rows0, lds0 + 2 * TILE);
       if (T > 1) issue(krsrc, k_srb, false, rows_v, lds0 + TILE);
@@ -402,11 +410,24 @@ __device__ __forceinline__ void attn_item(const AttnParams& p, char* smem, const
           prefetch_raw(t, raw);
         }
       };
-      first_raw(0, raw);
-      finish_rows(0, raw, rows0, nv0);
-      if (T > 1) { first_raw(1, raw); finish_rows(1, raw, rows_v, nv1); }
-      if (T > 2) { first_raw(2, raw); finish_rows(2, raw, rows_k, nv2); }
-      if (T > 3) first_raw(3, raw);
+      if constexpr (MODE == MODE_GATHER) {
+        // the list entries of the first four tiles are requested together (one memory round trip, not one per tile)
+        int raw0[NR], raw1[NR], raw2[NR];
+        prefetch_raw(0, raw0);
+        prefetch_raw(1, raw1);
+        prefetch_raw(2, raw2);
+        prefetch_raw(3, raw);
+        finish_rows(0, raw0, rows0, nv0);
+        finish_rows(1, raw1, rows_v, nv1);
+        finish_rows(2, raw2, rows_k, nv2);
+        nv1 = max(nv1, 0); nv2 = max(nv2, 0);
+      } else {
+        first_raw(0, raw);
+        finish_rows(0, raw, rows0, nv0);
+        if (T > 1) { first_raw(1, raw); finish_rows(1, raw, rows_v, nv1); }
+        if (T > 2) { first_raw(2, raw); finish_rows(2, raw, rows_k, nv2); }
+        if (T > 3) first_raw(3, raw);
+      }
       issue(krsrc, k_srb, false, rows0, lds0);
       if (!LSE_ONLY) issue(vrsrc, v_srb, true, rows0, lds0 + 2 * TILE);
       if (T > 1) issue(krsrc, k_srb, false, rows_v, lds0 + TILE);
