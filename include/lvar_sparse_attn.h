@@ -227,7 +227,8 @@ int lvar_block_sparse_attn_ws_fwd(lvar_tensor_t q, lvar_tensor_t k, lvar_tensor_
  * entry point allocates nothing and takes no memory beyond the inputs and outputs from the caller.  It has no
  * counterpart in the reference; it is for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments, results and balanced-launch
- * rule as lvar_block_sparse_attn_ws_fwd given a zeroed workspace of LVAR_STATIC_SCRATCH_BYTES.
+ * rule as lvar_block_sparse_attn_ws_fwd given a workspace of LVAR_STATIC_SCRATCH_BYTES; arguments are checked before the
+ * buffer is looked at, so a refused call has not touched it.
  * Limits: B * H * ceil(Lq / 128) (ceil(Lq / 64) for 64-row query blocks) <= LVAR_STATIC_MAX_QUERY_TILES and head_dim <= 128, else LVAR_ETOOBIG (larger
  * launches have enough query tiles to fill the chip: use lvar_block_sparse_attn_fwd).  All calls on one GPU share
  * that GPU's buffer: calls that overlap in time on one GPU (different streams or threads) race.
