@@ -278,22 +278,25 @@ static int launch_cs(const ColsumParams& p0, hipStream_t stream) {
   if (p.kv_group < 1) p.kv_group = 1;
   p.nkb = (p.Lk + 63) / 64;
   p.nkt = (p.Lk + 255) / 256;
-  // Ranges of query groups per key tile.  With fewer than four rounds of workgroups on the chip's resident slots
-  // (two per CU) the last, partly filled round costs as much as a full one: cut the query axis so that the rounds
-  // get shorter.  Cost model: rounds x (64-row stages per range + 3 stages' worth of fixed cost per workgroup).
+  // Ranges of query groups per key tile.  Workgroups are handed to the resident slots (two per compute unit) as slots
+  // fall free, so a launch takes about its total work spread over the slots plus a part of the longest workgroup, during
+  // which the chip drains.  More, shorter ranges shorten that tail and pay the fixed cost of a workgroup more often.
+  // In 64-row stages, fitted to launches of 0.06 .. 0.37 ms on 256 compute units:
+  //   cost = workgroups x (stages of a range + 1.5) / slots  +  0.4 x (stages of the longest range + 1.5)
   const int unit = (p.group_rows % 64 == 0) ? p.group_rows : (p.group_rows % 32 == 0 ? 2 * p.group_rows : 0);   // lcm(group_rows, 64)
   p.q_splits = 1;
   p.split_rows = ((p.Lq + 63) / 64) * 64 + (unit > 0 ? unit : 64);   // one range covers everything
   const int base_wg = p.B * p.H * p.nkt, slots = 2 * device_cus();
-  if (unit > 0 && slots > 0 && base_wg < 4 * slots) {
+  if (unit > 0 && slots > 0 && base_wg < 4 * slots) {   // longer launches: the tail is small whatever the cut
     const int units_total = (p.Lq + unit - 1) / unit;
-    int64_t best = -1;
+    double best = -1.0;
     for (int s = 1; s <= 8 && s <= units_total; s++) {
       const int rows = ((units_total + s - 1) / s) * unit;          // rows per range
       const int n = (p.Lq + rows - 1) / rows;                       // ranges that hold rows
-      const int64_t rounds = ((int64_t)base_wg * n + slots - 1) / slots;
-      const int64_t cost = rounds * ((rows + 63) / 64 + 3);
-      if (best < 0 || cost < best) { best = cost; p.q_splits = n; p.split_rows = rows; }
+      const int st_long = (std::min(rows, p.Lq) + 63) / 64, st_last = (p.Lq - (n - 1) * rows + 63) / 64;
+      const double work = (double)base_wg * ((n - 1) * (st_long + 1.5) + (st_last + 1.5)) / slots;
+      const double cost = work + 0.4 * (st_long + 1.5);
+      if (best < 0.0 || cost < best) { best = cost; p.q_splits = n; p.split_rows = rows; }
     }
   }
   p.total_wg = base_wg * p.q_splits;
