@@ -319,7 +319,7 @@ def run_hbm_workload(args, dev, wl):
         cn = torch.empty(B, H, G, dtype=torch.int32, device=dev)
         fn = lambda: lib.lvar_topk_token_lists(cs.data_ptr(), Lk, idx.data_ptr(), Lk, cn.data_ptr(), B * H * G, Lk, cnt, 0, stream)
         nbytes = B * H * G * (Lk * 4 + cnt * 4 + 4)
-        kernel, unit_desc = "topk_token_lists_kernel<24,512>", f"{B * H * G} rows x {Lk} fp32 scores, k = {cnt}"
+        kernel, unit_desc = f"topk_token_lists_kernel<{(Lk + 511) // 512},512>", f"{B * H * G} rows x {Lk} fp32 scores, k = {cnt}"
         fn()
         assert torch.equal(idx[..., :cnt].cpu(), oracle.topk_token_set(cs_cpu, cnt)), "top-k differs from the oracle"
         if not args.no_cpu_baseline:

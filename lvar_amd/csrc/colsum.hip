@@ -140,8 +140,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void colsum_kernel(const C
       acc[nt] = 0.f;
     }
     if (bsp) {
-#pragma unroll
-      for (int m = 16; m >= 1; m >>= 1) blk += __shfl_xor(blk, m);
+      blk = group_sum<32>(blk);
       if (lane == 0 && n0 < p.Lk) bsp[(int64_t)g * p.nkb + kblk] = blk;
     }
   };

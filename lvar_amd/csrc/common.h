@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace lvar {
 
@@ -41,6 +42,24 @@ __device__ __forceinline__ float xhalf_max(float x) {
 __device__ __forceinline__ float xhalf_sum(float x) {
   auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), false, false);
   return __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
+}
+
+// Sum over aligned groups of LANES lanes (8, 16 or 32), every lane of a group receiving the total: butterfly steps as
+// data-parallel-primitive moves (swap inside pairs, swap of pairs inside quads, mirror inside 8, mirror inside 16), which
+// pair the same partial sums as exchanges with lane^1, ^2, ^4, ^8 and so give the same bits, without the round trips
+// through the LDS crossbar that a shuffle costs.
+template <int LANES>
+__device__ __forceinline__ float group_sum(float x) {
+  static_assert(LANES == 8 || LANES == 16 || LANES == 32, "group size");
+  auto mv = [](float v, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, true));
+  };
+  x += mv(x, std::integral_constant<int, 0xB1>{});    // quad_perm [1,0,3,2]
+  x += mv(x, std::integral_constant<int, 0x4E>{});    // quad_perm [2,3,0,1]
+  x += mv(x, std::integral_constant<int, 0x141>{});   // row_half_mirror
+  if constexpr (LANES >= 16) x += mv(x, std::integral_constant<int, 0x140>{});   // row_mirror
+  if constexpr (LANES >= 32) x += __shfl_xor(x, 16, 64);
+  return x;
 }
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {

@@ -2,6 +2,7 @@
 // column sums, the cross-scale query-group remap fused with the local-run append, and the
 // compaction of a boolean mask into index lists.  All three are HBM/L2-bound integer work: one pass
 // (or a few L2-resident passes) over the rows, ballot/prefix compaction, no sorting.
+#include <utility>
 #include "common.h"
 #include "launch.h"
 
@@ -9,6 +10,27 @@ namespace lvar {
 
 __device__ __forceinline__ int lanes_below(unsigned long long bal, int lane) {
   return __builtin_popcountll(bal & ((1ull << lane) - 1ull));
+}
+
+// Inclusive scan over the 64 lanes of a wave with data-parallel-primitive moves (row shifts by 1, 2, 4, 8 inside the rows
+// of 16 lanes, then the last lane of row 0 / 2 broadcast into row 1 / 3 and the last lane of row 1 into rows 2 and 3):
+// six dependent vector instructions instead of six round trips through the LDS crossbar.  Lanes that a move does not
+// reach take the identity.  Lane 63 ends up with the reduction over the wave.
+template <class Op>
+__device__ __forceinline__ int wave_scan(int v, const int identity, Op op) {
+  v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x111, 0xf, 0xf, false));   // row_shr:1
+  v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x112, 0xf, 0xf, false));   // row_shr:2
+  v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x114, 0xf, 0xf, false));   // row_shr:4
+  v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x118, 0xf, 0xf, false));   // row_shr:8
+  v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x142, 0xa, 0xf, false));   // row_bcast:15 into rows 1 and 3
+  v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x143, 0xc, 0xf, false));   // row_bcast:31 into rows 2 and 3
+  return v;
+}
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_readlane(wave_scan((int)v, 0, [](int a, int b) { return (int)max((uint32_t)a, (uint32_t)b); }), 63);
+}
+__device__ __forceinline__ uint32_t wave_umin(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_readlane(wave_scan((int)v, -1, [](int a, int b) { return (int)min((uint32_t)a, (uint32_t)b); }), 63);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -27,10 +49,10 @@ constexpr int TOPK_BINS = 2048;
 constexpr int TOPK_CAND = 256;   // keys of the first pass's bin that are resolved by direct comparison
 
 template <int KPT, int NT>
-__global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kernel(const TopkListParams p) {
+__global__ __launch_bounds__(NT, (KPT >= 1 && KPT <= 24) ? 6 : 1) void topk_token_lists_kernel(const TopkListParams p) {
   constexpr int NW = NT / 64;
   __shared__ int hist[TOPK_BINS];
-  __shared__ uint32_t cand[TOPK_CAND];
+  __shared__ __attribute__((aligned(16))) uint32_t cand[TOPK_CAND];
   __shared__ int wsum[NW];
   __shared__ int sel[2];  // chosen bin, keys still wanted inside it
   __shared__ int ncand;
@@ -92,11 +114,8 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
   // would fall into a handful of bins of the first pass and the LDS atomics of a wave would serialise on them.  The
   // bits that the largest and the smallest key of the row have in common are therefore taken as known, and the
   // digits start at the first bit in which keys differ: `top` low bits are left to resolve, 11 at a time.
-#pragma unroll
-  for (int d = 32; d > 0; d >>= 1) {
-    kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d, 64));
-    kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, 64));
-  }
+  kmax = wave_umax(kmax);
+  kmin = wave_umin(kmin);
   if (lane == 0) { wgt[wave] = (int)kmax; weq[wave] = (int)kmin; }
   if (tid == 0) ncand = 0;
   __syncthreads();
@@ -123,12 +142,7 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
     const int btop = nbins - 1 - tid * bpt;
     int mine = 0;
     for (int e = 0; e < bpt; e++) mine += (btop - e >= 0) ? hist[btop - e] : 0;
-    int incl = mine;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int o = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += o;
-    }
+    const int incl = wave_scan(mine, 0, [](int a, int b) { return a + b; });
     if (lane == 63) wsum[wave] = incl;
     __syncthreads();
     int before = incl - mine;
@@ -170,10 +184,15 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
         if (tid < nc) {
           const uint32_t kt = cand[tid];
           int above = 0, at_or_above = 0;
-          for (int u = 0; u < nc; u++) {
-            const uint32_t ku = cand[u];
-            above += ku > kt;
-            at_or_above += ku >= kt;
+          // four candidates per LDS read (all lanes read the same address): the loop is bound by the latency of its reads
+          for (int u = 0; u < nc; u += 4) {
+            const u32x4 ku = *(const u32x4*)(cand + u);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const bool in = u + e < nc;
+              above += in && ku[e] > kt;
+              at_or_above += in && ku[e] >= kt;
+            }
           }
           if (above < want && want <= at_or_above) { sel[0] = (int)kt; sel[1] = want - above; }   // equal keys write equal values
         }
@@ -224,16 +243,24 @@ __global__ __launch_bounds__(NT, (KPT == 24) ? 6 : 1) void topk_token_lists_kern
   if (lane < fill) out[pos + lane] = ring[(head + lane) & 127];
 }
 
+// Keys per thread: every value up to 24 (a row of n keys takes ceil(n / 512) of them: no pass walks more than one
+// chunk of padding per wave), then 28 and 32; longer rows are re-read from L2 in every pass.
+template <int KPT>
+static bool topk_try(const TopkListParams& p, hipStream_t stream) {
+  if (p.n > 512 * KPT) return false;
+  hipLaunchKernelGGL((topk_token_lists_kernel<KPT, 512>), dim3(p.rows), dim3(512), 0, stream, p);
+  return true;
+}
+template <int... KPT>
+static bool topk_dispatch(const TopkListParams& p, hipStream_t stream, std::integer_sequence<int, KPT...>) {
+  return (topk_try<KPT + 1>(p, stream) || ...);
+}
+
 int launch_topk_token_lists(const TopkListParams& p, hipStream_t stream) {
   if (p.rows == 0) return LVAR_OK;
-  const dim3 grid(p.rows);
   // 512 threads per row keep a row of up to 16384 keys in registers (KPT keys per thread)
-  if (p.n <= 512 * 4) hipLaunchKernelGGL((topk_token_lists_kernel<4, 512>), grid, dim3(512), 0, stream, p);
-  else if (p.n <= 512 * 8) hipLaunchKernelGGL((topk_token_lists_kernel<8, 512>), grid, dim3(512), 0, stream, p);
-  else if (p.n <= 512 * 16) hipLaunchKernelGGL((topk_token_lists_kernel<16, 512>), grid, dim3(512), 0, stream, p);
-  else if (p.n <= 512 * 24) hipLaunchKernelGGL((topk_token_lists_kernel<24, 512>), grid, dim3(512), 0, stream, p);
-  else if (p.n <= 512 * 32) hipLaunchKernelGGL((topk_token_lists_kernel<32, 512>), grid, dim3(512), 0, stream, p);
-  else hipLaunchKernelGGL((topk_token_lists_kernel<0, 512>), grid, dim3(512), 0, stream, p);
+  if (!topk_dispatch(p, stream, std::make_integer_sequence<int, 24>{}) && !topk_try<28>(p, stream) && !topk_try<32>(p, stream))
+    hipLaunchKernelGGL((topk_token_lists_kernel<0, 512>), dim3(p.rows), dim3(512), 0, stream, p);
   return hipGetLastError() == hipSuccess ? LVAR_OK : LVAR_ELAUNCH;
 }
 

@@ -90,8 +90,7 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const WinScoreParams
       float dot = 0.f;
 #pragma unroll
       for (int e = 0; e < 4; e++) dot += bf16_lo(kv[u][e]) * qv[2 * e] + bf16_hi(kv[u][e]) * qv[2 * e + 1];
-#pragma unroll
-      for (int m = LPR >> 1; m > 0; m >>= 1) dot += __shfl_xor(dot, m, 64);
+      dot = group_sum<LPR>(dot);
       if (l == 0 && j < span) {
         sc[j] = (n >= 0 && n < p.Lk) ? dot * p.scale : pad;
         wm[j] = 0;
