@@ -271,6 +271,16 @@ def test_topk_token_lists_matches_oracle_set():
     for k in (1, 832, 2060, 4121):
         idx, cnt = ops.topk_token_lists(x.cuda(), k)
         assert torch.equal(idx[..., :k].cpu(), oracle.topk_token_set(x, k)), k
+    # row lengths on both sides of every keys-per-thread step of the kernel (512 keys per step up to 12288, then 14336
+    # and 16384, beyond that the rows are re-read): ragged last chunks, a whole chunk of padding, ties through the cut
+    for n in (1, 63, 64, 65, 511, 512, 513, 1024, 1025, 4607, 4608, 4609, 10240, 10752, 10753, 12288, 12289, 14336, 14337,
+              16384, 16385):
+        x = torch.rand(3, n, generator=g)
+        x[1] = torch.randint(0, 7, (n,), generator=g).float()              # heavy ties
+        x[2] = -x[2]
+        for k in sorted({1, max(1, n // 5), n}):
+            idx, cnt = ops.topk_token_lists(x.cuda(), k)
+            assert torch.equal(idx[..., :k].cpu(), oracle.topk_token_set(x, k)), (n, k)
     x = torch.rand(2, 2, 3, 500, generator=g)
     idx, _ = ops.topk_token_lists(x.cuda(), 64, order="value")
     assert torch.equal(idx[..., :64].cpu().long(), torch.topk(x, 64, dim=-1).indices)   # distinct values: same order
