@@ -289,6 +289,41 @@ def test_topk_token_lists_matches_oracle_set():
 
 
 @pytest.mark.gpu
+def test_list_kernels_seeded_sweep():
+    """Seeded sweep of the two list builders against the oracle, bit-exact: row lengths around the chunk and
+    keys-per-thread steps, value distributions with heavy ties / one binade / both signs, every k regime; masks of
+    every density with count rounding."""
+    import random
+    import oracle
+    from lvar_amd import sparse_attn_ops as ops
+    rnd = random.Random(7)
+    g = torch.Generator().manual_seed(7)
+    for it in range(120):
+        rows = rnd.randint(1, 4)
+        n = rnd.choice([1, 2, 7, 63, 64, 65, 129, 511, 512, 513, 777, 2047, 2049, 4121, 6425, 10521, 13000, 16384, 17000])
+        kind = rnd.random()
+        x = torch.rand(rows, n, generator=g) ** rnd.choice([1, 4, 9])
+        if kind < 0.2:
+            x = (x * rnd.choice([3, 8, 50])).round()            # heavy ties
+        elif kind < 0.3:
+            x = 0.0181 + x * 1e-4                                 # one binade
+        elif kind < 0.4:
+            x = x - 0.5                                           # both signs
+        k = rnd.choice([0, 1, max(1, n // 5), max(1, n // 2), n])
+        idx, cnt = ops.topk_token_lists(x.cuda(), k)
+        assert torch.equal(idx[..., :k].cpu(), oracle.topk_token_set(x, k)), (it, rows, n, k)
+    for it in range(80):
+        b, h, m = rnd.randint(1, 3), rnd.randint(1, 4), rnd.randint(1, 6)
+        n = rnd.choice([1, 2, 5, 63, 64, 65, 100, 192, 300, 1000, 2049])
+        dens = rnd.choice([0.0, 0.05, 0.3, 0.9, 1.0])
+        mult = rnd.choice([1, 2, 7, 64, 192])
+        mask = torch.rand(b, h, m, n, generator=g) < dens
+        idx, cnt = ops.mask_to_indices(mask.cuda(), mult, rnd.choice([1, 8, 192]))
+        c_ref, i_ref = oracle.mask_to_lists(mask, mult)
+        assert torch.equal(cnt.cpu(), c_ref) and torch.equal(idx[..., :n].cpu(), i_ref), (it, b, h, m, n, dens, mult)
+
+
+@pytest.mark.gpu
 def test_remap_concat_lists_matches_oracle():
     import oracle
     from lvar_amd import sparse_attn_ops as ops
